@@ -1,0 +1,155 @@
+#!/usr/bin/env python3
+"""Throughput of the CRF-CTC decode on one MI355X, next to the CPU path.
+
+One step = one `openfish_decode_gpu` call (backward scan, beam search, forward +
+posterior scan, sequence stage, copy of moves/sequence/qstring to the host) over
+one batch of synthetic scores that already sit in HBM.  The default workload is
+the headline configuration: hac model (state_len 4, 256 states, C = 1024),
+T = 1666, N = 512 chunks, fp16 scores drawn N(0, 2) (+1 on the dropped blank
+column), beam width 32, beam cut 100, blank score 2.0.
+
+Prints ONE JSON line:
+  value      chunks decoded per second (wall clock around the K timed calls)
+  roofline   the longest-running kernel: algorithmic bytes / mean device time
+             (HIP events recorded by the library on the kernel's own stream)
+  stages     every kernel's mean device time and algorithmic GB/s
+  cpu_baseline  the CPU path timed on this host on a bounded sample of the same tensor
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+WORKLOADS = {
+    # name: (state_len, T, N, stress, q_scale, q_shift)
+    "fast": (3, 1666, 512, False, 0.97, -1.8),
+    "hac": (4, 1666, 512, False, 0.95, -0.2),
+    "sup": (5, 1666, 256, False, 0.95, 0.5),
+    "hac_stress": (4, 1666, 1024, True, 0.95, -0.2),
+}
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(state_len, T, N):
+    """bytes each kernel has to move at least once, per launch"""
+    S = 4 ** state_len
+    C = 4 * S
+    scores = T * C * 2
+    vec = (T + 1) * S * 4
+    return {
+        "bwd": N * (scores + vec),                    # read scores, write bwd
+        "fwd_post": N * (scores + 2 * vec),           # read scores + bwd, write post
+        "beam": N * (scores + T * S * 4 + (T + 1) * 32 * 2 * 2 + 5 * T),  # rows, beam slots out+in, states+moves
+        "sequence": N * (9 * 4 * T + 5 * T + 16 * T + 8 * T + 2 * T),  # gathers, states/moves, qual, probs, text
+    }
+
+
+def cpu_baseline(s16, state_len, opt_kw, sample_chunks):
+    """the reference CPU path (oracle/_ref when it was built, else the oracle port) on the
+    first `sample_chunks` chunks of the same tensor; median of 3 after one warm-up"""
+    from oracle import crf_oracle as O
+    T = s16.shape[0]
+    sub = np.ascontiguousarray(s16[:, :sample_chunks, :]).astype(np.float32)
+    cores = min(os.cpu_count() or 1, 16, sample_chunks)
+    if O.have_ref():
+        kind = "reference"
+        run = lambda: O.ref_decode(sub, state_len, opt_kw, nthreads=cores)  # noqa: E731
+    else:
+        kind = "port"
+        run = lambda: O.decode(sub, state_len, opt_kw, nthreads=cores, dump=False)  # noqa: E731
+    run()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    sec = statistics.median(times)
+    return {"value": sample_chunks / sec, "unit": "chunks/s", "cores": cores, "kind": kind,
+            "sample": "first %d chunks of the same tensor, T=%d, fp32 copy of the fp16 values, "
+                      "median of 3 calls of openfish_decode_cpu (%.3f s each)" % (sample_chunks, T, sec)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="hac", choices=sorted(WORKLOADS))
+    ap.add_argument("--chunks", type=int, default=0, help="override N")
+    ap.add_argument("--scan-mode", default="precise", choices=("precise", "fast"))
+    ap.add_argument("--cpu-sample", type=int, default=64, help="chunks timed on the CPU path (0 = skip)")
+    ap.add_argument("--seed", type=int, default=20251125)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this decoder runs on one GPU; chunks are independent, so more GPUs means "
+                 "one process and one batch shard per GPU (no collective). Run with --gpus 1.")
+
+    from openfish_amd import api, synth
+    if api.device_count() < 1:
+        sys.exit("bench.py: no HIP device visible")
+
+    state_len, T, N, stress, q_scale, q_shift = WORKLOADS[a.workload]
+    if a.chunks:
+        N = a.chunks
+    S = 4 ** state_len
+    C = 4 * S
+    scale = synth.stress_scale(N) if stress else None
+    s16 = synth.crf_scores(T, N, state_len, seed=a.seed, chunk_scale=scale, threads=16)
+
+    api.set_scan_mode(a.scan_mode == "fast")
+    opt = api.DECODER_INIT(q_scale=q_scale, q_shift=q_shift)
+    scores = api.upload_scores_to_hip(s16)
+    gpubuf = api.GpuBuf(T, N, state_len)
+
+    for _ in range(a.warmup):
+        api.openfish_decode_gpu(T, N, C, scores, state_len, opt, gpubuf)
+    api.lib().openfish_amd_sync()
+    per_stage = {k: [] for k in api.STAGES}
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        api.openfish_decode_gpu(T, N, C, scores, state_len, opt, gpubuf)
+        for k, v in gpubuf.timings().items():
+            per_stage[k].append(v)
+    api.lib().openfish_amd_sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = 1e3 * wall / a.steps
+
+    need = algorithmic_bytes(state_len, T, N)
+    stages = {}
+    for k in ("bwd", "fwd_post", "beam", "sequence"):
+        ms = statistics.mean(per_stage[k])
+        stages[k] = {"ms": round(ms, 4), "algorithmic_GB": round(need[k] / 1e9, 4),
+                     "GBps": round(need[k] / 1e9 / (ms / 1e3), 1)}
+    stages["device_total_ms"] = round(statistics.mean(per_stage["total"]), 4)
+    scan_ms = stages["bwd"]["ms"] + stages["fwd_post"]["ms"]
+    scan_gbs = (need["bwd"] + need["fwd_post"]) / 1e9 / (scan_ms / 1e3)
+    stages["scan_plus_posterior"] = {"ms": round(scan_ms, 4), "GBps": round(scan_gbs, 1),
+                                     "frac_of_hbm_peak": round(scan_gbs / HBM_PEAK_GBS, 4)}
+    dominant = max(("bwd", "fwd_post", "beam", "sequence"), key=lambda k: stages[k]["ms"])
+    roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(stages[dominant]["GBps"] / HBM_PEAK_GBS, 4), "traffic": None}
+
+    opt_kw = dict(beam_cut=100.0, blank_score=2.0, q_shift=q_shift, q_scale=q_scale)
+    cpu = cpu_baseline(s16, state_len, opt_kw, min(a.cpu_sample, N)) if a.cpu_sample > 0 else None
+
+    print(json.dumps({
+        "metric": "CRF chunks decoded/sec at %s (%d states, T=%d, N=%d); achieved HBM GB/s" % (a.workload, S, T, N),
+        "value": round(N / (ms_per_step / 1e3), 1), "unit": "chunks/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: state_len %d, S=%d, C=%d fp16 TNC, T=%d, N=%d, beam 32, beam_cut 100, blank 2.0"
+                               % (a.workload, state_len, S, C, T, N),
+                   "scan_mode": a.scan_mode, "seed": a.seed},
+        "roofline": roofline, "stages": stages, "cpu_baseline": cpu,
+    }))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,139 @@
+/*
+ * Stage-level C-ABI of the MI355X decoder: the same work openfish_decode_gpu
+ * does, one stage at a time, on caller-provided device buffers.  Used by
+ * parity tests and benchmarks; plain pointers and sizes only.
+ *
+ * Every function works on the current device, is synchronous unless stated,
+ * and follows the library's error convention (message on stderr, exit).
+ */
+#ifndef OPENFISH_AMD_H
+#define OPENFISH_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "openfish.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- device helpers (reference src/decode_hip.h:34-54, src/decode_hip.hip:220-346) ---- */
+
+/* reference set_device_hip, src/decode_hip.hip:220-226 */
+void set_device_hip(int device);
+/* reference upload_scores_to_hip, src/decode_hip.hip:228-244: host half [T][N][C] -> new device buffer */
+void *upload_scores_to_hip(const int T, const int N, const int C, const void *scores_TNC);
+/* reference free_scores_hip, src/decode_hip.hip:246-252 */
+void free_scores_hip(void *scores_TNC_gpu);
+/* reference write_gpubuf_hip, src/decode_hip.hip:254-346: dumps bwd_NTC, post_NTC, qual_data,
+ * base_probs, total_probs of a gpubuf as <name>.blob into the current directory */
+void write_gpubuf_hip(const uint64_t T, const uint64_t N, const int state_len,
+                      const openfish_gpubuf_t *gpubuf);
+
+/* raw device memory for harnesses that have no HIP binding of their own */
+void *openfish_amd_malloc(size_t bytes);
+void openfish_amd_free(void *dev);
+void openfish_amd_memcpy_h2d(void *dev, const void *host, size_t bytes);
+void openfish_amd_memcpy_d2h(void *host, const void *dev, size_t bytes);
+void openfish_amd_memset(void *dev, int value, size_t bytes);
+void openfish_amd_sync(void);
+/* number of visible devices; 0 when there is none (never exits) */
+int openfish_amd_device_count(void);
+
+/* ---- stages ---- */
+
+/*
+ * Backward scan (reference backward_scan src/decode_cpu.c:13-52, GPU twin
+ * bwd_scan src/scan_hip.hip:9-58).  scores: device half [T][N][C], C = 4*S.
+ * bwd: device fp32 [N][T+1][S], row T is zero.
+ */
+void openfish_amd_bwd_scan(int T, int N, int C, const void *scores, int state_len, float stay_score,
+                           float *bwd);
+
+/*
+ * Forward scan fused with the per-time-step posterior softmax (reference
+ * forward_scan + softmax src/decode_cpu.c:54-147, GPU twin fwd_post_scan
+ * src/scan_hip.hip:60-200).  post: device fp32 [N][T+1][S].
+ */
+void openfish_amd_fwd_post_scan(int T, int N, int C, const void *scores, int state_len,
+                                float stay_score, const float *bwd, float *post);
+
+/*
+ * Beam search and traceback (reference beam_search_cpu src/beam_search.c:117-439).
+ * Reads scores and bwd, fills gpubuf->beam_vector, gpubuf->states (int32 [N][T],
+ * the full k-mer state of the traced path) and gpubuf->moves.
+ */
+void openfish_amd_beam_search(int T, int N, int C, const void *scores, int state_len,
+                              const openfish_opt_t *options, const float *bwd,
+                              const openfish_gpubuf_t *gpubuf);
+
+/*
+ * Per-block quality, base calls and phred string (reference src/beam_search.c:441-496
+ * and generate_sequence_cpu src/beam_search.c:49-99).  Reads post, gpubuf->states and
+ * gpubuf->moves; fills gpubuf->qual_data, base_probs, total_probs, sequence, qstring
+ * and reduces gpubuf->states to the emitted base (state & 3) as the reference does.
+ */
+void openfish_amd_sequence(int T, int N, int state_len, const openfish_opt_t *options,
+                           const float *post, const openfish_gpubuf_t *gpubuf);
+
+/*
+ * Beam search + sequence stage fed with external bwd/post tensors (device fp32
+ * [N][T+1][S]); outputs as openfish_decode_gpu.  This is the entry the bit-exact
+ * acceptance test uses with the CPU path's own tensors.
+ */
+void openfish_amd_decode_from_tensors(int T, int N, int C, const void *scores, int state_len,
+                                      const openfish_opt_t *options, const float *bwd,
+                                      const float *post, const openfish_gpubuf_t *gpubuf,
+                                      uint8_t **moves, char **sequence, char **qstring);
+
+/* ---- measurement ---- */
+
+enum openfish_amd_stage {
+    OPENFISH_AMD_STAGE_BWD = 0,   /* backward scan kernel */
+    OPENFISH_AMD_STAGE_FWD = 1,   /* forward + posterior kernel */
+    OPENFISH_AMD_STAGE_BEAM = 2,  /* beam search + traceback kernel */
+    OPENFISH_AMD_STAGE_SEQ = 3,   /* quality + sequence kernel */
+    OPENFISH_AMD_STAGE_TOTAL = 4, /* first launch to last kernel end, device side */
+    OPENFISH_AMD_STAGE_COUNT = 5
+};
+
+/*
+ * Device-side durations in milliseconds (HIP events on the streams the kernels
+ * ran on) of the most recent openfish_decode_gpu call on this gpubuf.  Writes
+ * min(n, OPENFISH_AMD_STAGE_COUNT) values and returns that count.
+ */
+int openfish_amd_last_timings(const openfish_gpubuf_t *gpubuf, float *ms, int n);
+
+/*
+ * Test hook.  Bit 0 makes the beam search replay every stay/step merge serially in
+ * the CPU path's order, the route it otherwise takes only after a CRC collision
+ * between beam hashes; outputs must be identical with and without it.
+ */
+void openfish_amd_set_debug_flags(int flags);
+
+/*
+ * Arithmetic of the two scans.  0 (default): exp/log in double with the CPU path's
+ * sequence of fp32 roundings (reference src/decode_cpu.c:45-49,104-108), so that bwd
+ * and the posterior reproduce the CPU tensors.  1: hardware fp32 exp/log, faster,
+ * bwd within 2 ulp; a last-bit difference of a scan value of magnitude 4096..8192 is a
+ * 5e-4 relative difference of the posterior built from it.  Process-wide.
+ */
+void openfish_amd_set_scan_mode(int fast);
+
+/*
+ * The 49 miss-probability thresholds behind the phred characters for one
+ * (q_scale, q_shift): char(x) = 83 - #{j : x >= thr[j]} equals
+ * (char)(33.5f + clamp(-10*log10f(x)*q_scale + q_shift, 1, 50)) of the reference
+ * (src/beam_search.c:92-97) for every x in [0,1].  Host-only; needs no device.
+ */
+void openfish_amd_phred_table(float q_scale, float q_shift, float *thr49);
+
+/* library build tag, e.g. "openfish-amd gfx950" */
+const char *openfish_amd_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* OPENFISH_AMD_H */

@@ -1,0 +1,256 @@
+"""Python mirror of the openfish C API, bound with ctypes to
+openfish_amd/libopenfish_amd.so (the same objects as lib/libopenfish.a).
+
+The functions keep the C names and argument meaning (include/openfish/openfish.h,
+include/openfish/openfish_amd.h).  There is no fallback of any kind: if the
+shared library has not been built the import of this module fails, and any
+device error makes the C library print a message and exit the process, as the
+reference library does.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libopenfish_amd.so")
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "%s is missing: build it with `make` at the repository root "
+        "(or __graft_entry__.build()); there is no CPU fallback" % LIB_PATH)
+
+_L = C.CDLL(LIB_PATH)
+
+STAGES = ("bwd", "fwd_post", "beam", "sequence", "total")
+
+
+class openfish_opt_t(C.Structure):
+    """reference include/openfish/openfish.h:29-37"""
+    _fields_ = [("beam_width", C.c_size_t), ("beam_cut", C.c_float), ("blank_score", C.c_float),
+                ("q_shift", C.c_float), ("q_scale", C.c_float), ("temperature", C.c_float),
+                ("move_pad", C.c_bool)]
+
+
+class openfish_gpubuf_t(C.Structure):
+    """reference include/openfish/openfish.h:16-27"""
+    _fields_ = [("bwd_NTC", C.c_void_p), ("post_NTC", C.c_void_p), ("moves", C.c_void_p),
+                ("sequence", C.c_void_p), ("qstring", C.c_void_p), ("beam_vector", C.c_void_p),
+                ("states", C.c_void_p), ("qual_data", C.c_void_p), ("base_probs", C.c_void_p),
+                ("total_probs", C.c_void_p)]
+
+
+def DECODER_INIT(**kw):
+    """{32, 100.0, 2.0, 0.0, 1.0, 1.0, false} with keyword overrides"""
+    o = openfish_opt_t(32, 100.0, 2.0, 0.0, 1.0, 1.0, False)
+    for k, v in kw.items():
+        setattr(o, k, v)
+    return o
+
+
+_vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
+_optp, _bufp = C.POINTER(openfish_opt_t), C.POINTER(openfish_gpubuf_t)
+_pp = C.POINTER(C.c_void_p)
+
+_SIGS = {
+    "openfish_gpubuf_init": (_bufp, [_i, _i, _i]),
+    "openfish_gpubuf_free": (None, [_bufp]),
+    "openfish_decode_gpu": (None, [_i, _i, _i, _vp, _i, _optp, _bufp, _pp, _pp, _pp]),
+    "openfish_rotary_emb_gpu": (None, [_vp, _vp, _vp] + [_i] * 8),
+    "openfish_decode_cpu": (None, [_i, _i, _i, _i, _vp, _i, _optp, _pp, _pp, _pp]),
+    "openfish_rotary_emb_cpu": (None, [_vp, _vp, _vp] + [_i] * 9),
+    "get_openfish_log_level": (_i, []),
+    "set_openfish_log_level": (None, [_i]),
+    "set_device_hip": (None, [_i]),
+    "upload_scores_to_hip": (_vp, [_i, _i, _i, _vp]),
+    "free_scores_hip": (None, [_vp]),
+    "write_gpubuf_hip": (None, [C.c_uint64, C.c_uint64, _i, _bufp]),
+    "openfish_amd_malloc": (_vp, [_sz]),
+    "openfish_amd_free": (None, [_vp]),
+    "openfish_amd_memcpy_h2d": (None, [_vp, _vp, _sz]),
+    "openfish_amd_memcpy_d2h": (None, [_vp, _vp, _sz]),
+    "openfish_amd_memset": (None, [_vp, _i, _sz]),
+    "openfish_amd_sync": (None, []),
+    "openfish_amd_device_count": (_i, []),
+    "openfish_amd_bwd_scan": (None, [_i, _i, _i, _vp, _i, _f, _vp]),
+    "openfish_amd_fwd_post_scan": (None, [_i, _i, _i, _vp, _i, _f, _vp, _vp]),
+    "openfish_amd_beam_search": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _bufp]),
+    "openfish_amd_sequence": (None, [_i, _i, _i, _optp, _vp, _bufp]),
+    "openfish_amd_decode_from_tensors": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _vp, _bufp, _pp, _pp, _pp]),
+    "openfish_amd_last_timings": (_i, [_bufp, C.POINTER(C.c_float), _i]),
+    "openfish_amd_set_debug_flags": (None, [_i]),
+    "openfish_amd_set_scan_mode": (None, [_i]),
+    "openfish_amd_phred_table": (None, [_f, _f, C.POINTER(C.c_float)]),
+    "openfish_amd_version": (C.c_char_p, []),
+}
+
+EXPORTS = tuple(_SIGS)
+
+for _name, (_res, _args) in _SIGS.items():
+    _fn = getattr(_L, _name)  # AttributeError here means the library lacks a declared symbol
+    _fn.restype = _res
+    _fn.argtypes = _args
+
+_libc = C.CDLL(None)
+_libc.free.argtypes = [C.c_void_p]
+
+
+def lib():
+    return _L
+
+
+def device_count():
+    return int(_L.openfish_amd_device_count())
+
+
+class DeviceBuffer:
+    """a device allocation owned by Python"""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        self.ptr = _L.openfish_amd_malloc(self.nbytes)
+
+    @classmethod
+    def from_host(cls, array):
+        a = np.ascontiguousarray(array)
+        b = cls(a.nbytes)
+        _L.openfish_amd_memcpy_h2d(b.ptr, a.ctypes.data, a.nbytes)
+        return b
+
+    def to_host(self, dtype, shape):
+        out = np.empty(shape, dtype)
+        assert out.nbytes <= self.nbytes
+        _L.openfish_amd_memcpy_d2h(out.ctypes.data, self.ptr, out.nbytes)
+        return out
+
+    def fill(self, byte):
+        _L.openfish_amd_memset(self.ptr, byte, self.nbytes)
+
+    def free(self):
+        if self.ptr:
+            _L.openfish_amd_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _device_to_host(ptr, dtype, shape):
+    out = np.empty(shape, dtype)
+    _L.openfish_amd_memcpy_d2h(out.ctypes.data, ptr, out.nbytes)
+    return out
+
+
+def _take(ptr, N, T):
+    """copy one malloc'd [N][T] byte buffer returned by the C API and free it"""
+    a = np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_uint8)), shape=(N, T)).copy()
+    _libc.free(ptr)
+    return a
+
+
+class GpuBuf:
+    """openfish_gpubuf_init / openfish_gpubuf_free"""
+
+    def __init__(self, T, N, state_len):
+        self.T, self.N, self.state_len = T, N, state_len
+        self.S = 4 ** state_len
+        self.handle = _L.openfish_gpubuf_init(T, N, state_len)
+
+    def free(self):
+        if self.handle:
+            _L.openfish_gpubuf_free(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+    def tensor(self, name, T=None, N=None):
+        """host copy of one device tensor of the gpubuf"""
+        T = T or self.T
+        N = N or self.N
+        f = self.handle.contents
+        shapes = {
+            "bwd_NTC": (np.float32, (N, T + 1, self.S)), "post_NTC": (np.float32, (N, T + 1, self.S)),
+            "moves": (np.uint8, (N, T)), "sequence": (np.uint8, (N, T)), "qstring": (np.uint8, (N, T)),
+            "states": (np.int32, (N, T)), "qual_data": (np.float32, (N, T, 4)),
+            "base_probs": (np.float32, (N, T)), "total_probs": (np.float32, (N, T)),
+            "beam_vector": (np.uint16, (N, T + 1, 32)),
+        }
+        dt, shp = shapes[name]
+        return _device_to_host(getattr(f, name), dt, shp)
+
+    def timings(self):
+        """device-side milliseconds of the stages of the last openfish_decode_gpu call"""
+        ms = (C.c_float * len(STAGES))()
+        n = _L.openfish_amd_last_timings(self.handle, ms, len(STAGES))
+        return {STAGES[k]: float(ms[k]) for k in range(n)}
+
+
+def openfish_decode_gpu(T, N, Cc, scores_dev, state_len, options, gpubuf):
+    """returns (moves, sequence, qstring) as uint8 [N][T] host arrays"""
+    mv, sq, qs = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    _L.openfish_decode_gpu(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), gpubuf.handle,
+                           C.byref(mv), C.byref(sq), C.byref(qs))
+    return _take(mv, N, T), _take(sq, N, T), _take(qs, N, T)
+
+
+def openfish_amd_decode_from_tensors(T, N, Cc, scores_dev, state_len, options, bwd_dev, post_dev, gpubuf):
+    mv, sq, qs = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    _L.openfish_amd_decode_from_tensors(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options),
+                                        _ptr(bwd_dev), _ptr(post_dev), gpubuf.handle,
+                                        C.byref(mv), C.byref(sq), C.byref(qs))
+    return _take(mv, N, T), _take(sq, N, T), _take(qs, N, T)
+
+
+def openfish_amd_bwd_scan(T, N, Cc, scores_dev, state_len, stay_score, bwd_dev):
+    _L.openfish_amd_bwd_scan(T, N, Cc, _ptr(scores_dev), state_len, stay_score, _ptr(bwd_dev))
+
+
+def openfish_amd_fwd_post_scan(T, N, Cc, scores_dev, state_len, stay_score, bwd_dev, post_dev):
+    _L.openfish_amd_fwd_post_scan(T, N, Cc, _ptr(scores_dev), state_len, stay_score, _ptr(bwd_dev), _ptr(post_dev))
+
+
+def openfish_amd_beam_search(T, N, Cc, scores_dev, state_len, options, bwd_dev, gpubuf):
+    _L.openfish_amd_beam_search(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), _ptr(bwd_dev), gpubuf.handle)
+
+
+def openfish_amd_sequence(T, N, state_len, options, post_dev, gpubuf):
+    _L.openfish_amd_sequence(T, N, state_len, C.byref(options), _ptr(post_dev), gpubuf.handle)
+
+
+def openfish_rotary_emb_gpu(x_dev, sin_dev, cos_dev, batch_size, seqlen, nheads, head_dim, rotary_half,
+                            stride_batch, stride_seq, stride_head):
+    _L.openfish_rotary_emb_gpu(_ptr(x_dev), _ptr(sin_dev), _ptr(cos_dev), batch_size, seqlen, nheads,
+                               head_dim, rotary_half, stride_batch, stride_seq, stride_head)
+
+
+def upload_scores_to_hip(scores_half):
+    """host fp16 [T][N][C] -> DeviceBuffer (reference upload_scores_to_hip)"""
+    a = np.ascontiguousarray(scores_half, dtype=np.float16)
+    return DeviceBuffer.from_host(a)
+
+
+def phred_table(q_scale, q_shift):
+    thr = (C.c_float * 49)()
+    _L.openfish_amd_phred_table(q_scale, q_shift, thr)
+    return np.array(thr[:], dtype=np.float32)
+
+
+def set_scan_mode(fast):
+    _L.openfish_amd_set_scan_mode(1 if fast else 0)
+
+
+def set_debug_flags(flags):
+    _L.openfish_amd_set_debug_flags(int(flags))
+
+
+def _ptr(x):
+    if isinstance(x, DeviceBuffer):
+        return x.ptr
+    return x

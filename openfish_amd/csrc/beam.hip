@@ -1,0 +1,573 @@
+// Beam search over one chunk per workgroup, gfx950.
+//
+// A workgroup is two wavefronts.  Wave 1 streams the rows the search needs
+// (scores[t] as fp16 and bwd[t+1] as fp32) from HBM into an LDS ring, several
+// rows ahead; wave 0 runs the search with the 32-wide beam resident in
+// registers/LDS.  The two communicate through two LDS counters (rows ready /
+// rows consumed), so the search never waits on a dependent HBM gather.
+//
+// Wave 0 lane layout: lane = i + 32*h holds beam element i (mirrored in both
+// halves) and the step candidates with new base 2h and 2h+1; lanes < 32 also hold
+// the stay candidate.  Candidate order is the CPU path's: steps 4i+b, then stays.
+// The search reproduces the CPU path (reference src/beam_search.c:117-439) to the
+// bit: same fp32 operation order, double-precision log-sum-exp for merges, the
+// same cut-off bisection, first-come compaction and final best-to-slot-0 swap.
+// Instead of sorting, the cut-off uses wave ballots and population counts, and
+// survivors are ranked with ballot prefix counts.
+//
+// Stay/step merging: a stay of element i merges with the step (j, b_i) whose hash
+// crc(hash_j, b_i) equals hash_i.  The 2-bit CRC update is a bijection of the
+// 32-bit state, so this is the same as hash_j == crc^-1(hash_i, b_i): every lane
+// inverts its own hash once and compares it with the 32 previous hashes.
+#include <hip/hip_runtime.h>
+
+#include <cfloat>
+
+#include "kernels.h"
+
+namespace {
+
+constexpr int kW = OFK_BEAM_WIDTH;
+constexpr uint32_t kPoly = 0x82f63b78u;
+constexpr uint32_t kSeed = 0x12345678u;
+
+constexpr uint32_t crc_bits(uint32_t crc, uint32_t bits, int n) {
+    for (int i = 0; i < n; ++i) {
+        const uint32_t feed = (bits ^ crc) & 1u;
+        crc >>= 1;
+        if (feed) crc ^= kPoly;
+        bits >>= 1;
+    }
+    return crc;
+}
+// CRC-32C is linear over GF(2): two update steps are (crc >> 2) xor a table entry chosen
+// by the two low bits of crc ^ bits, and the entry for 3 is the xor of those for 1 and 2.
+constexpr uint32_t kTab1 = crc_bits(1u, 0u, 2);
+constexpr uint32_t kTab2 = crc_bits(2u, 0u, 2);
+static_assert(crc_bits(3u, 0u, 2) == (kTab1 ^ kTab2), "crc linearity");
+static_assert((kTab1 >> 30) == 1u && (kTab2 >> 30) == 2u, "top bits identify the table entry");
+
+__device__ __forceinline__ uint32_t crc_tab(uint32_t x) {
+    return ((0u - (x & 1u)) & kTab1) ^ ((0u - ((x >> 1) & 1u)) & kTab2);
+}
+__device__ __forceinline__ uint32_t crc2(uint32_t crc, uint32_t base) {
+    return (crc >> 2) ^ crc_tab((crc ^ base) & 3u);
+}
+// the hash h with crc2(h, base) == crc
+__device__ __forceinline__ uint32_t crc2_inverse(uint32_t crc, uint32_t base) {
+    const uint32_t k = crc >> 30;
+    return ((crc ^ crc_tab(k)) << 2) | (k ^ base);
+}
+__device__ __forceinline__ uint32_t crc32_word(uint32_t crc, uint32_t word) {
+    for (int i = 0; i < 16; ++i) {
+        crc = crc2(crc, word & 3u);
+        word >>= 2;
+    }
+    return crc;
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float lane_f(float x, int lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), lane));
+}
+__device__ __forceinline__ uint32_t lane_u(uint32_t x, int lane) {
+    return (uint32_t)__builtin_amdgcn_readlane((int)x, lane);
+}
+__device__ __forceinline__ float wave_max(float x) {
+    x = fmaxf(x, dpp<0x128>(x));
+    x = fmaxf(x, dpp<0x124>(x));
+    x = fmaxf(x, dpp<0x122>(x));
+    x = fmaxf(x, dpp<0x121>(x));
+    return fmaxf(fmaxf(lane_f(x, 0), lane_f(x, 16)), fmaxf(lane_f(x, 32), lane_f(x, 48)));
+}
+__device__ __forceinline__ int wave_sum_i(int x) {
+    x += __builtin_amdgcn_update_dpp(0, x, 0x128, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, 0x124, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, 0x122, 0xF, 0xF, true);
+    x += __builtin_amdgcn_update_dpp(0, x, 0x121, 0xF, 0xF, true);
+    return __builtin_amdgcn_readlane(x, 0) + __builtin_amdgcn_readlane(x, 16) +
+           __builtin_amdgcn_readlane(x, 32) + __builtin_amdgcn_readlane(x, 48);
+}
+__device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
+__device__ __forceinline__ int popc64(uint64_t x) { return __builtin_popcountll(x); }
+
+__device__ __forceinline__ void wave_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Hand-over of LDS rows between the two waves of a workgroup.  The fences name the
+// local address space only: they wait for outstanding LDS operations, not for the
+// global loads and stores each wave keeps in flight.
+__device__ __forceinline__ void publish(int *flag, int value) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __hip_atomic_store(flag, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ int observe(int *flag) {
+    const int v = __hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    return v;
+}
+
+// log(e^x + e^y) with the correction evaluated in double and dropped for gaps >= 17
+// (reference src/beam_search.c:43-47)
+__device__ __forceinline__ float log_sum_exp(float x, float y) {
+    const float gap = fabsf(x - y);
+    const float top = x > y ? x : y;
+    const double corr = gap < 17.0f ? log(1.0 + exp(-(double)gap)) : 0.0;
+    return (float)((double)top + corr);
+}
+
+__device__ __forceinline__ uint32_t float_key(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+__device__ __forceinline__ float key_float(uint32_t k) {
+    return __uint_as_float(k ^ ((k >> 31) ? 0x80000000u : 0xFFFFFFFFu));
+}
+
+template <int BYTES>
+struct Vec;
+template <>
+struct Vec<4> { typedef uint32_t type; };
+template <>
+struct Vec<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <>
+struct Vec<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+
+// one wave's share of a row of ROW_BYTES bytes: lane l owns vectors (i*64 + l)
+template <int ROW_BYTES>
+struct RowRegs {
+    static constexpr int kPer = ROW_BYTES / 64;
+    static constexpr int kVec = kPer >= 16 ? 16 : kPer;
+    static constexpr int kCnt = kPer / kVec;
+    typedef typename Vec<kVec>::type V;
+    V v[kCnt];
+    __device__ __forceinline__ void load(const char *row, int lane) {
+#pragma unroll
+        for (int i = 0; i < kCnt; ++i) v[i] = *reinterpret_cast<const V *>(row + (size_t)(i * 64 + lane) * kVec);
+    }
+    __device__ __forceinline__ void store(char *row, int lane) const {
+#pragma unroll
+        for (int i = 0; i < kCnt; ++i) *reinterpret_cast<V *>(row + (size_t)(i * 64 + lane) * kVec) = v[i];
+    }
+};
+
+template <int S>
+struct BeamCfg {
+    static constexpr int kBits = S == 64 ? 6 : S == 256 ? 8 : 10;
+    static constexpr int kLdsRows = S >= 1024 ? 3 : 6;  // LDS ring depth
+    static constexpr int kRegRows = S >= 1024 ? 3 : 6;  // rows in flight in registers (3 or 6)
+    static constexpr int kTraceBlock = 128;             // time steps staged per traceback block
+};
+
+struct BeamShared {
+    uint32_t hash[kW];
+    int32_t state[kW];
+    float score[kW];
+    uint32_t meta[kW];       // prev | stay << 5
+    float cand[5 * kW];      // candidate scores: steps at 4i+b, stays at 128+i
+    uint8_t owner[4 * kW];   // which stay claimed a step during a merge
+    int ready;               // rows stored by the loader wave
+    int consumed;            // rows the search wave is done with
+};
+
+template <int S>
+__global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ scores,
+                                                   const float *__restrict__ bwd,
+                                                   ofk_beam_slot_t *__restrict__ beam,
+                                                   int32_t *__restrict__ states, uint8_t *__restrict__ moves,
+                                                   int T, int N, float log_cut, float stay, int flags) {
+    using Cfg = BeamCfg<S>;
+    constexpr int BITS = Cfg::kBits;
+    constexpr int LR = Cfg::kLdsRows;
+    constexpr int RR = Cfg::kRegRows;
+    constexpr int TB = Cfg::kTraceBlock;
+
+    __shared__ __attribute__((aligned(16))) _Float16 row_s[LR][4 * S];
+    __shared__ __attribute__((aligned(16))) float row_b[LR][S];
+    __shared__ __attribute__((aligned(16))) BeamShared sh;
+    __shared__ __attribute__((aligned(16))) ofk_beam_slot_t trace[TB][kW];
+    __shared__ int32_t trace_state[TB];
+    __shared__ uint8_t trace_move[TB];
+
+    const int n = blockIdx.x;
+    const int lane = threadIdx.x & 63;
+    const size_t row_stride = (size_t)N * 4 * S;
+    const _Float16 *sc_n = scores + (size_t)n * 4 * S;
+    const float *bw_n = bwd + (size_t)n * (size_t)(T + 1) * S;
+
+    if (threadIdx.x == 0) {
+        sh.ready = 0;
+        sh.consumed = 0;
+    }
+    __syncthreads();
+
+    if (threadIdx.x >= 64) {
+        // ---- loader wave: row t = (scores[t], bwd[t+1]) into ring slot t % LR ----
+        // The ring is spelled out as named registers (not an array indexed by a loop that
+        // also contains the spin wait) so that every row stays in VGPRs.
+        RowRegs<8 * S> s0, s1, s2, s3, s4, s5;
+        RowRegs<4 * S> g0, g1, g2, g3, g4, g5;
+        auto fetch = [&](RowRegs<8 * S> &rs, RowRegs<4 * S> &rb, int t) {
+            if (t < T) {
+                rs.load(reinterpret_cast<const char *>(sc_n + (size_t)t * row_stride), lane);
+                rb.load(reinterpret_cast<const char *>(bw_n + (size_t)(t + 1) * S), lane);
+            }
+        };
+        auto hand_over = [&](RowRegs<8 * S> &rs, RowRegs<4 * S> &rb, int t) {
+            if (t < T) {
+                while (t - observe(&sh.consumed) >= LR) __builtin_amdgcn_s_sleep(1);
+                const int slot = t % LR;
+                rs.store(reinterpret_cast<char *>(row_s[slot]), lane);
+                rb.store(reinterpret_cast<char *>(row_b[slot]), lane);
+                fetch(rs, rb, t + RR);
+                publish(&sh.ready, t + 1);
+            }
+        };
+        fetch(s0, g0, 0);
+        fetch(s1, g1, 1);
+        fetch(s2, g2, 2);
+        if constexpr (RR == 6) {
+            fetch(s3, g3, 3);
+            fetch(s4, g4, 4);
+            fetch(s5, g5, 5);
+        }
+        for (int t0 = 0; t0 < T; t0 += RR) {
+            hand_over(s0, g0, t0);
+            hand_over(s1, g1, t0 + 1);
+            hand_over(s2, g2, t0 + 2);
+            if constexpr (RR == 6) {
+                hand_over(s3, g3, t0 + 3);
+                hand_over(s4, g4, t0 + 4);
+                hand_over(s5, g5, t0 + 5);
+            }
+        }
+        return;
+    }
+
+    // ---- search wave ----
+    const int i = lane & 31;
+    const int h = lane >> 5;
+    const uint64_t below = (((uint64_t)1 << i) - 1) * 0x100000001ull;  // elements < i, both halves
+
+    // seeding: the 32 best states of bwd[0] in ascending state order (src/beam_search.c:151-175)
+    {
+        constexpr int PER = S / 64;
+        float v[PER];
+        uint32_t key[PER];
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            v[j] = bw_n[j * 64 + lane];
+            key[j] = float_key(v[j]);
+        }
+        uint32_t prefix = 0;  // largest K with #{key >= K} >= 32, i.e. the 32nd largest value
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t trial = prefix | (1u << bit);
+            int c = 0;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) c += key[j] >= trial ? 1 : 0;
+            if (wave_sum_i(c) >= kW) prefix = trial;
+        }
+        const float thr = key_float(prefix);
+        if (lane < kW) {
+            sh.hash[lane] = 0;
+            sh.state[lane] = 0;
+            sh.score[lane] = 0.f;
+            sh.meta[lane] = 0;
+        }
+        wave_fence();
+        int taken = 0;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const bool ok = v[j] >= thr;
+            const uint64_t m = ballot(ok);
+            const int rank = taken + popc64(m & (((uint64_t)1 << lane) - 1));
+            if (ok && rank < kW) {
+                const int s = j * 64 + lane;
+                sh.hash[rank] = crc32_word(kSeed, (uint32_t)s);
+                sh.state[rank] = s;
+            }
+            taken += popc64(m);
+        }
+        wave_fence();
+    }
+    uint32_t hash = sh.hash[i];
+    int state = sh.state[i];
+    float score = 0.f;
+    int w = kW;
+    ofk_beam_slot_t *bv = beam + (size_t)n * (size_t)(T + 1) * kW;
+    if (lane < kW) bv[lane] = (ofk_beam_slot_t)state;
+
+    for (int t = 0; t < T; ++t) {
+        while (observe(&sh.ready) <= t) __builtin_amdgcn_s_sleep(1);
+        const int slot = t % LR;
+        const _Float16 *rs = row_s[slot];
+        const float *rb = row_b[slot];
+
+        const bool valid = i < w;
+        const int lo4 = (state << 2) & (S - 1);
+        const int top = state >> (BITS - 2);
+        const int b0 = 2 * h;
+        const float r0 = (float)rs[4 * (lo4 + b0) + top];
+        const float r1 = (float)rs[4 * (lo4 + b0 + 1) + top];
+        const float2 g01 = *reinterpret_cast<const float2 *>(&rb[lo4 + b0]);
+        const float gst = rb[state];
+        float c0 = (score + r0) + g01.x;
+        float c1 = (score + r1) + g01.y;
+        float cs = (score + stay) + gst;
+        const uint32_t h0 = crc2(hash, (uint32_t)b0);
+        const uint32_t h1 = crc2(hash, (uint32_t)b0 + 1u);
+
+        // which previous element j has hash_j == crc^-1(hash_i, last base of i)
+        uint32_t match;
+        {
+            const uint32_t want = crc2_inverse(hash, (uint32_t)state & 3u);
+            const uint4 *hp = reinterpret_cast<const uint4 *>(&sh.hash[16 * h]);
+            uint32_t m = 0;
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const uint4 x = hp[qd];
+                m |= (x.x == want ? 1u : 0u) << (4 * qd);
+                m |= (x.y == want ? 1u : 0u) << (4 * qd + 1);
+                m |= (x.z == want ? 1u : 0u) << (4 * qd + 2);
+                m |= (x.w == want ? 1u : 0u) << (4 * qd + 3);
+            }
+            m <<= 16 * h;
+            m |= (uint32_t)__shfl_xor((int)m, 32);
+            const uint32_t live = w >= 32 ? 0xFFFFFFFFu : ((1u << w) - 1u);
+            match = valid ? (m & live) : 0u;
+        }
+
+        if (ballot(match != 0) != 0) {
+            // merge stays with the step spelling the same sequence (src/beam_search.c:281-316)
+            sh.cand[4 * i + b0] = c0;
+            sh.cand[4 * i + b0 + 1] = c1;
+            const bool mine = h == 0 && match != 0;
+            const int j = __builtin_ctz(match | 0x80000000u);
+            const int target = 4 * (j & 31) + (state & 3);
+            if (h == 0) sh.cand[4 * kW + i] = cs;
+            if (mine) sh.owner[target] = (uint8_t)i;
+            wave_fence();
+            bool odd = false;
+            float other = 0.f;
+            if (mine) {
+                other = sh.cand[target];
+                odd = (match & (match - 1)) != 0 || sh.owner[target] != (uint8_t)i;
+            }
+            if (ballot(odd) != 0 || (flags & 1)) {
+                // A stay with several equal hashes, or a step claimed by two stays (only
+                // possible after a CRC collision): replay the merges one by one in the
+                // CPU path's order.
+                wave_fence();
+                if (lane == 0) {
+                    for (int a = 0; a < w; ++a) {
+                        const uint32_t ha = sh.hash[a];
+                        const int base = sh.state[a] & 3;
+                        const int si = 4 * kW + a;
+                        for (int b = 0; b < w; ++b) {
+                            if (crc2(sh.hash[b], (uint32_t)base) != ha) continue;
+                            const int st = 4 * b + base;
+                            const float folded = log_sum_exp(sh.cand[si], sh.cand[st]);
+                            if (sh.cand[si] > sh.cand[st]) {
+                                sh.cand[si] = folded;
+                                sh.cand[st] = -FLT_MAX;
+                            } else {
+                                sh.cand[st] = folded;
+                                sh.cand[si] = -FLT_MAX;
+                            }
+                        }
+                    }
+                }
+                wave_fence();
+                if (h == 0) cs = sh.cand[4 * kW + i];
+            } else {
+                if (mine) {
+                    const float folded = log_sum_exp(cs, other);
+                    if (cs > other) {
+                        cs = folded;
+                        sh.cand[target] = -FLT_MAX;
+                    } else {
+                        cs = -FLT_MAX;
+                        sh.cand[target] = folded;
+                    }
+                }
+                wave_fence();
+            }
+            c0 = sh.cand[4 * i + b0];
+            c1 = sh.cand[4 * i + b0 + 1];
+        }
+
+        // cut-off (src/beam_search.c:320-381)
+        const bool has_stay = valid && h == 0;
+        float best = -FLT_MAX;
+        if (valid) best = fmaxf(c0, c1);
+        if (has_stay) best = fmaxf(best, cs);
+        best = wave_max(best);
+
+        float cut = best - log_cut;
+        uint64_t k0 = ballot(valid && c0 >= cut), k1 = ballot(valid && c1 >= cut), ks = ballot(has_stay && cs >= cut);
+        int kept = popc64(k0) + popc64(k1) + popc64(ks);
+        if (kept > kW) {
+            float lo = cut, hi = best;
+            int guesses = 1;
+            while ((kept > kW || kept < (kW * 8) / 10) && guesses < 10) {
+                if (kept > kW) {
+                    lo = cut;
+                    cut = (cut + hi) / 2.0f;
+                } else {
+                    hi = cut;
+                    cut = (cut + lo) / 2.0f;
+                }
+                k0 = ballot(valid && c0 >= cut);
+                k1 = ballot(valid && c1 >= cut);
+                ks = ballot(has_stay && cs >= cut);
+                kept = popc64(k0) + popc64(k1) + popc64(ks);
+                ++guesses;
+            }
+            if (guesses == 10) {
+                cut = hi;
+                k0 = ballot(valid && c0 >= cut);
+                k1 = ballot(valid && c1 >= cut);
+                ks = ballot(has_stay && cs >= cut);
+                kept = popc64(k0) + popc64(k1) + popc64(ks);
+            }
+            if (kept > kW) kept = kW;
+        }
+
+        // survivors in candidate order: steps (i, b) by i then b, then stays by i
+        {
+            const int before = popc64(k0 & below) + popc64(k1 & below);
+            const uint32_t k0lo = (uint32_t)k0, k1lo = (uint32_t)k1;
+            const int same = h == 0 ? 0 : (int)((k0lo >> i) & 1u) + (int)((k1lo >> i) & 1u);
+            const bool keep0 = (k0 >> lane) & 1u, keep1 = (k1 >> lane) & 1u, keeps = (ks >> lane) & 1u;
+            const int rank0 = before + same;
+            const int rank1 = rank0 + (keep0 ? 1 : 0);
+            const int ranks = popc64(k0) + popc64(k1) + popc64(ks & below);
+            wave_fence();
+            if (keep0 && rank0 < kW) {
+                sh.hash[rank0] = h0;
+                sh.state[rank0] = lo4 + b0;
+                sh.score[rank0] = c0;
+                sh.meta[rank0] = (uint32_t)i;
+            }
+            if (keep1 && rank1 < kW) {
+                sh.hash[rank1] = h1;
+                sh.state[rank1] = lo4 + b0 + 1;
+                sh.score[rank1] = c1;
+                sh.meta[rank1] = (uint32_t)i;
+            }
+            if (keeps && ranks < kW) {
+                sh.hash[ranks] = hash;
+                sh.state[ranks] = state;
+                sh.score[ranks] = cs;
+                sh.meta[ranks] = (uint32_t)i | 32u;
+            }
+            wave_fence();
+        }
+        w = kept;
+        uint32_t meta = 0;
+        if (i < w) {
+            hash = sh.hash[i];
+            state = sh.state[i];
+            score = sh.score[i];
+            meta = sh.meta[i];
+        } else {
+            state = 0;
+            score = 0.f;
+        }
+
+        // last block: the best survivor goes to slot 0 (src/beam_search.c:398-414)
+        if (t == T - 1) {
+            const bool in = i < w;
+            const float top_score = wave_max(in ? score : -FLT_MAX);
+            const uint64_t at = ballot(in && h == 0 && score == top_score);
+            const int arg = (top_score > -FLT_MAX && at != 0) ? __builtin_ctzll(at) : 0;
+            if (arg != 0) {
+                const uint32_t hash0 = lane_u(hash, 0), hasha = lane_u(hash, arg);
+                const int st0 = (int)lane_u((uint32_t)state, 0), sta = (int)lane_u((uint32_t)state, arg);
+                const float sc0 = lane_f(score, 0), sca = lane_f(score, arg);
+                const uint32_t me0 = lane_u(meta, 0), mea = lane_u(meta, arg);
+                if (i == 0) { hash = hasha; state = sta; score = sca; meta = mea; }
+                if (i == arg) { hash = hash0; state = st0; score = sc0; meta = me0; }
+                wave_fence();
+                if (lane == 0 || lane == arg) {
+                    sh.hash[i] = hash;
+                    sh.state[i] = state;
+                }
+                wave_fence();
+            }
+        }
+
+        // drop the guide term again and persist the slot (src/beam_search.c:417-427)
+        if (i < w) {
+            score = score - rb[state];
+            if (h == 0)
+                bv[(size_t)(t + 1) * kW + i] =
+                    (ofk_beam_slot_t)((uint32_t)state | ((meta & 31u) << 10) | ((meta >> 5) << 15));
+        }
+        publish(&sh.consumed, t + 1);
+    }
+
+    // ---- traceback from slot 0 of the last block (src/beam_search.c:432-439) ----
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    int32_t *st_out = states + (size_t)n * T;
+    uint8_t *mv_out = moves + (size_t)n * T;
+    int cursor = 0;
+    for (int hi_t = T; hi_t > 0; hi_t -= TB) {
+        const int lo_t = hi_t > TB ? hi_t - TB : 0;  // rows lo_t+1 .. hi_t
+        const int rows = hi_t - lo_t;
+        const uint4 *src = reinterpret_cast<const uint4 *>(bv + (size_t)(lo_t + 1) * kW);
+        uint4 *dst = reinterpret_cast<uint4 *>(&trace[0][0]);
+        for (int x = lane; x < rows * 4; x += 64) dst[x] = src[x];  // 64 bytes per row
+        wave_fence();
+        for (int r = rows - 1; r >= 0; --r) {
+            const uint32_t e = trace[r][cursor];
+            if (lane == 0) {
+                trace_state[r] = (int32_t)(e & 1023u);
+                trace_move[r] = (e >> 15) ? 0 : 1;
+            }
+            cursor = (int)((e >> 10) & 31u);
+        }
+        wave_fence();
+        for (int x = lane; x < rows; x += 64) {
+            st_out[lo_t + x] = trace_state[x];
+            mv_out[lo_t + x] = (lo_t + x == 0) ? (uint8_t)1 : trace_move[x];
+        }
+        wave_fence();
+    }
+}
+
+template <int S>
+int launch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
+                uint8_t *moves, int T, int N, float log_cut, float stay, int flags, hipStream_t st) {
+    hipLaunchKernelGGL((beam_kernel<S>), dim3(N), dim3(128), 0, st, static_cast<const _Float16 *>(scores),
+                       bwd, beam, states, moves, T, N, log_cut, stay, flags);
+    return (int)hipGetLastError();
+}
+
+int g_beam_flags = 0;
+
+}  // namespace
+
+extern "C" void ofk_set_beam_flags(int flags) { g_beam_flags = flags; }
+
+extern "C" int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
+                               uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
+                               void *stream) {
+    if (!scores || !bwd || !beam || !states || !moves || T < 1 || N < 1) return OFK_BAD_ARGS;
+    if ((reinterpret_cast<uintptr_t>(scores) | reinterpret_cast<uintptr_t>(bwd) | reinterpret_cast<uintptr_t>(beam)) & 15u)
+        return OFK_BAD_ARGS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (state_len) {
+        case 3: return launch_beam<64>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, st);
+        case 4: return launch_beam<256>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, st);
+        case 5: return launch_beam<1024>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, st);
+        default: return OFK_BAD_ARGS;
+    }
+}

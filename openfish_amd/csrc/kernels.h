@@ -1,0 +1,53 @@
+/*
+ * Launchers of the gfx950 kernels, callable from C.  Each returns 0 on success,
+ * a hipError_t value if the launch failed, or OFK_BAD_ARGS if the arguments do
+ * not fit what the kernel assumes (nothing is launched in that case).
+ */
+#ifndef OPENFISH_AMD_KERNELS_H
+#define OPENFISH_AMD_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OFK_BAD_ARGS (-1)
+#define OFK_BEAM_WIDTH 32
+
+/* one persisted beam slot, 16 bit: state[9:0] | prev[14:10] | stay[15] */
+typedef uint16_t ofk_beam_slot_t;
+
+/* 0 (default): scans reproduce the CPU path's double exp/log and fp32 roundings;
+ * 1: scans use the hardware fp32 exp/log (faster, last-bit differences). */
+void ofk_set_scan_fast(int on);
+int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, float stay,
+                 void *stream);
+int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N,
+                      int state_len, float stay, void *stream);
+int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
+                    uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
+                    void *stream);
+/* bit 0: replay every stay/step merge one by one in CPU order (the path otherwise taken
+ * only after a hash collision); results must not change.  For tests. */
+void ofk_set_beam_flags(int flags);
+/* Phred characters run from '"' (34, q = 1) to 'S' (83, q = 50).  thr[j] is the smallest
+ * miss probability x whose character is at most 82 - j (2.0f if no x in [0,1] reaches it),
+ * so that char(x) = 83 - #{j : x >= thr[j]}. */
+#define OFK_PHRED_STEPS 49
+typedef struct {
+    float thr[OFK_PHRED_STEPS];
+} ofk_phred_table_t;
+
+int ofk_sequence(const float *post, int32_t *states, const uint8_t *moves, float *qual_data,
+                 float *base_probs, float *total_probs, char *sequence, char *qstring, int T, int N,
+                 int state_len, const ofk_phred_table_t *phred, void *stream);
+int ofk_rotary_emb(void *x, const float *sin_buf, const float *cos_buf, int batch, int seqlen,
+                   int nheads, int rotary_half, long stride_batch, long stride_seq, long stride_head,
+                   void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

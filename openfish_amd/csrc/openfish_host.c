@@ -1,0 +1,460 @@
+/*
+ * Host side of the MI355X decoder: the public openfish entry points and the
+ * stage-level C-ABI, in C, above the kernel launchers of kernels.h.
+ *
+ * One decode is   bwd scan -> { beam search || fwd+posterior scan } -> sequence.
+ * The beam search needs only scores and bwd, the posterior only feeds the quality
+ * stage (reference src/beam_search.c:193,450), so the two run on two streams and
+ * share the device.  Errors follow the reference convention (reference
+ * src/hip_utils.h:11-28, src/error.h:44-72): message on stderr, then exit.
+ */
+#include <errno.h>
+#include <float.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <hip/hip_runtime_api.h>
+
+#include <openfish/openfish.h>
+#include <openfish/openfish_amd.h>
+#include <openfish/openfish_error.h>
+
+#include "kernels.h"
+
+/* ---- logging (reference src/error.c:33-41) -------------------------------- */
+
+static enum openfish_log_level_opt g_log_level = OPENFISH_LOG_VERB;
+
+enum openfish_log_level_opt get_openfish_log_level(void) { return g_log_level; }
+void set_openfish_log_level(enum openfish_log_level_opt level) { g_log_level = level; }
+
+void openfish_log_emit(enum openfish_log_level_opt need, const char *tag, const char *colour,
+                       const char *func, const char *file, int line, int where, const char *fmt, ...) {
+    if (g_log_level < need) return;
+    va_list ap;
+    if (colour) fprintf(stderr, "[%s::%s]%s ", func, tag, colour);
+    else fprintf(stderr, "[%s] %s: ", tag, func);
+    va_start(ap, fmt);
+    vfprintf(stderr, fmt, ap);
+    va_end(ap);
+    if (colour) fputs("\033[0m", stderr);
+    if (where) fprintf(stderr, " At %s:%d", file, line);
+    fputc('\n', stderr);
+}
+
+/* ---- error convention ------------------------------------------------------ */
+
+#define HIP_OK(call)                                                                              \
+    do {                                                                                          \
+        hipError_t e_ = (call);                                                                   \
+        if (e_ != hipSuccess) {                                                                   \
+            fprintf(stderr, "HIP error: %s, in file: %s, line number: %d\n", hipGetErrorString(e_), \
+                    __FILE__, __LINE__);                                                          \
+            exit(1);                                                                              \
+        }                                                                                         \
+    } while (0)
+
+static void die(const char *what) {
+    OPENFISH_ERROR("%s", what);
+    exit(EXIT_FAILURE);
+}
+
+static void launch_ok(int rc, const char *kernel) {
+    if (rc == 0) return;
+    if (rc == OFK_BAD_ARGS) fprintf(stderr, "openfish: %s: arguments do not fit the kernel (shape, alignment or state_len)\n", kernel);
+    else fprintf(stderr, "HIP error: %s, launching %s\n", hipGetErrorString((hipError_t)rc), kernel);
+    exit(1);
+}
+
+static void *host_alloc(size_t bytes) {
+    void *p = malloc(bytes ? bytes : 1);
+    if (!p) {
+        fprintf(stderr, "openfish: out of host memory (%zu bytes)\n", bytes);
+        exit(EXIT_FAILURE);
+    }
+    return p;
+}
+
+/* ---- gpubuf ---------------------------------------------------------------- */
+
+#define OFA_MAGIC 0x6f66616d64677075ull /* "ofamdgpu" */
+
+enum { EV_JOIN, EV_START, EV_BWD_END, EV_BEAM_START, EV_BEAM_END, EV_FWD_END, EV_SEQ_START, EV_SEQ_END, EV_COUNT };
+
+typedef struct {
+    openfish_gpubuf_t pub; /* first: the pointer handed to callers is this struct */
+    unsigned long long magic;
+    int T, N, state_len;
+    void *slab;            /* one device allocation behind all pub fields */
+    unsigned char *h_out;  /* pinned staging for moves | sequence | qstring */
+    hipStream_t s_main, s_side;
+    hipEvent_t ev[EV_COUNT];
+    float ms[OPENFISH_AMD_STAGE_COUNT];
+    int timed;
+    ofk_phred_table_t phred; /* thresholds for (phred_shift, phred_scale) */
+    float phred_shift, phred_scale;
+    int phred_valid;
+} ofa_gpubuf_t;
+
+static size_t round_up(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static int states_of(int state_len) { return 1 << (2 * state_len); }
+
+static void check_state_len(int state_len) {
+    if (state_len < 3 || state_len > 5) die("state_len must be 3, 4 or 5 (64, 256 or 1024 states)");
+}
+
+openfish_gpubuf_t *openfish_gpubuf_init(const int T, const int N, const int state_len) {
+    check_state_len(state_len);
+    if (T < 1 || N < 1) die("gpubuf: T and N must be positive");
+    const size_t S = (size_t)states_of(state_len), nt = (size_t)N * (size_t)T;
+    const size_t tens = sizeof(float) * (size_t)N * (size_t)(T + 1) * S;
+    ofa_gpubuf_t *g = (ofa_gpubuf_t *)host_alloc(sizeof *g);
+    memset(g, 0, sizeof *g);
+    g->magic = OFA_MAGIC;
+    g->T = T;
+    g->N = N;
+    g->state_len = state_len;
+
+    /* field sizes as in the reference (src/decode_hip.hip:24-48) except beam_vector,
+     * whose slots are 2 bytes here */
+    const size_t sz[10] = {tens, tens, nt, nt, nt,
+                           sizeof(ofk_beam_slot_t) * (size_t)N * OFK_BEAM_WIDTH * (size_t)(T + 1),
+                           sizeof(int32_t) * nt, sizeof(float) * 4 * nt, sizeof(float) * nt, sizeof(float) * nt};
+    size_t total = 0;
+    for (int i = 0; i < 10; ++i) total += round_up(sz[i]);
+    HIP_OK(hipMalloc(&g->slab, total));
+    unsigned char *p = (unsigned char *)g->slab;
+    void **field[10] = {(void **)&g->pub.bwd_NTC, (void **)&g->pub.post_NTC, (void **)&g->pub.moves,
+                        (void **)&g->pub.sequence, (void **)&g->pub.qstring, &g->pub.beam_vector,
+                        &g->pub.states, (void **)&g->pub.qual_data, (void **)&g->pub.base_probs,
+                        (void **)&g->pub.total_probs};
+    for (int i = 0; i < 10; ++i) {
+        *field[i] = p;
+        p += round_up(sz[i]);
+    }
+    HIP_OK(hipHostMalloc((void **)&g->h_out, 3 * nt, hipHostMallocDefault));
+    HIP_OK(hipStreamCreateWithFlags(&g->s_main, hipStreamNonBlocking));
+    HIP_OK(hipStreamCreateWithFlags(&g->s_side, hipStreamNonBlocking));
+    for (int i = 0; i < EV_COUNT; ++i) HIP_OK(hipEventCreate(&g->ev[i]));
+    return &g->pub;
+}
+
+void openfish_gpubuf_free(openfish_gpubuf_t *gpubuf) {
+    ofa_gpubuf_t *g = (ofa_gpubuf_t *)gpubuf;
+    if (!g) return;
+    if (g->magic != OFA_MAGIC) die("gpubuf was not created by openfish_gpubuf_init");
+    for (int i = 0; i < EV_COUNT; ++i) HIP_OK(hipEventDestroy(g->ev[i]));
+    HIP_OK(hipStreamDestroy(g->s_main));
+    HIP_OK(hipStreamDestroy(g->s_side));
+    HIP_OK(hipHostFree(g->h_out));
+    HIP_OK(hipFree(g->slab));
+    g->magic = 0;
+    free(g);
+}
+
+static ofa_gpubuf_t *checked(const openfish_gpubuf_t *gpubuf, int T, int N, int state_len) {
+    ofa_gpubuf_t *g = (ofa_gpubuf_t *)gpubuf;
+    if (!g || g->magic != OFA_MAGIC) die("gpubuf was not created by openfish_gpubuf_init");
+    if (state_len != g->state_len || (size_t)N * (size_t)(T + 1) > (size_t)g->N * (size_t)(g->T + 1) ||
+        (size_t)N * (size_t)T > (size_t)g->N * (size_t)g->T)
+        die("batch shape exceeds the shape the gpubuf was created for");
+    return g;
+}
+
+static void check_scores(int T, int N, int C, const void *scores, int state_len, const openfish_opt_t *opt) {
+    check_state_len(state_len);
+    if (T < 1 || N < 1) die("T and N must be positive");
+    if (C != 4 * states_of(state_len)) die("C must be 4 * 4^state_len (one score per state and dropped base)");
+    if (!scores) die("scores_TNC is NULL");
+    if (!opt) die("options is NULL");
+}
+
+static float log_beam_cut(const openfish_opt_t *opt) {
+    /* reference src/beam_search.c:135 */
+    return opt->beam_cut > 0.0f ? logf(opt->beam_cut) : FLT_MAX;
+}
+
+/* ---- phred thresholds -------------------------------------------------------
+ *
+ * The quality character of a base is char(x) = (char)(33.5f + clamp(-10*log10f(x)*scale
+ * + shift, 1, 50)) of its miss probability x = 1 - base_prob/total_prob (reference
+ * src/beam_search.c:92-97).  log10f is a libm routine whose last bit a device routine
+ * cannot be relied on to reproduce, but char(x) only steps 49 times over [0,1]: the
+ * thresholds are located here by bisection over the float bit patterns with this
+ * host's log10f, the neighbourhood of each is checked for monotonicity, and the
+ * kernel compares x against them.
+ */
+
+static int phred_char(float x, float scale, float shift) {
+    volatile float v = -10.0f * log10f(x);
+    volatile float q = v * scale;
+    q = q + shift;
+    if (q > 50.0f) q = 50.0f;
+    if (q < 1.0f) q = 1.0f;
+    return (int)(char)(33.5f + q);
+}
+
+static float bits_float(uint32_t b) {
+    float f;
+    memcpy(&f, &b, sizeof f);
+    return f;
+}
+
+static void build_phred_table(ofk_phred_table_t *tab, float scale, float shift) {
+    const uint32_t one = 0x3f800000u; /* 1.0f; bit patterns of [0,1] are ordered like the values */
+    for (int j = 0; j < OFK_PHRED_STEPS; ++j) {
+        const int limit = 82 - j;
+        if (phred_char(1.0f, scale, shift) > limit) {
+            tab->thr[j] = 2.0f; /* never reached on [0,1] */
+            continue;
+        }
+        uint32_t lo = 0, hi = one; /* char(lo) > limit >= char(hi) */
+        if (phred_char(0.0f, scale, shift) <= limit) hi = 0;
+        while (hi - lo > 1 && hi != 0) {
+            const uint32_t mid = lo + (hi - lo) / 2;
+            if (phred_char(bits_float(mid), scale, shift) <= limit) hi = mid;
+            else lo = mid;
+        }
+        tab->thr[j] = bits_float(hi);
+        for (uint32_t d = 1; d <= 64; ++d) {
+            const int below = hi >= d ? phred_char(bits_float(hi - d), scale, shift) : 127;
+            const int above = hi + d <= one ? phred_char(bits_float(hi + d), scale, shift) : 0;
+            if (below <= limit || above > limit)
+                die("phred character is not monotone in the miss probability near a threshold");
+        }
+    }
+}
+
+void openfish_amd_phred_table(float q_scale, float q_shift, float *thr49) {
+    ofk_phred_table_t tab;
+    build_phred_table(&tab, q_scale, q_shift);
+    memcpy(thr49, tab.thr, sizeof tab.thr);
+}
+
+static const ofk_phred_table_t *phred_for(ofa_gpubuf_t *g, const openfish_opt_t *opt) {
+    if (!g->phred_valid || g->phred_shift != opt->q_shift || g->phred_scale != opt->q_scale) {
+        build_phred_table(&g->phred, opt->q_scale, opt->q_shift);
+        g->phred_shift = opt->q_shift;
+        g->phred_scale = opt->q_scale;
+        g->phred_valid = 1;
+    }
+    return &g->phred;
+}
+
+/* ---- decode ---------------------------------------------------------------- */
+
+static void fetch_outputs(ofa_gpubuf_t *g, int T, int N, uint8_t **moves, char **sequence, char **qstring) {
+    const size_t nt = (size_t)N * (size_t)T;
+    *moves = (uint8_t *)host_alloc(nt);
+    *sequence = (char *)host_alloc(nt);
+    *qstring = (char *)host_alloc(nt);
+    HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_main));
+    HIP_OK(hipMemcpyAsync(g->h_out + nt, g->pub.sequence, nt, hipMemcpyDeviceToHost, g->s_main));
+    HIP_OK(hipMemcpyAsync(g->h_out + 2 * nt, g->pub.qstring, nt, hipMemcpyDeviceToHost, g->s_main));
+    HIP_OK(hipStreamSynchronize(g->s_main));
+    memcpy(*moves, g->h_out, nt);
+    memcpy(*sequence, g->h_out + nt, nt);
+    memcpy(*qstring, g->h_out + 2 * nt, nt);
+}
+
+/* order the library's streams after everything already queued on the null stream */
+static void join_null_stream(ofa_gpubuf_t *g) {
+    HIP_OK(hipEventRecord(g->ev[EV_JOIN], 0));
+    HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_JOIN], 0));
+}
+
+void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC, const int state_len,
+                         const openfish_opt_t *options, const openfish_gpubuf_t *gpubuf, uint8_t **moves,
+                         char **sequence, char **qstring) {
+    check_scores(T, N, C, scores_TNC, state_len, options);
+    ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
+    const float stay = options->blank_score; /* as the reference GPU path, src/decode_hip.hip:120 */
+    OPENFISH_LOG_TRACE("scores tensor dim: %d, %d, %d", T, N, C);
+
+    join_null_stream(g);
+    HIP_OK(hipEventRecord(g->ev[EV_START], g->s_main));
+    launch_ok(ofk_bwd_scan(scores_TNC, g->pub.bwd_NTC, T, N, state_len, stay, g->s_main), "bwd_scan");
+    HIP_OK(hipEventRecord(g->ev[EV_BWD_END], g->s_main));
+
+    HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BWD_END], 0));
+    HIP_OK(hipEventRecord(g->ev[EV_BEAM_START], g->s_side));
+    launch_ok(ofk_beam_search(scores_TNC, g->pub.bwd_NTC, (ofk_beam_slot_t *)g->pub.beam_vector,
+                              (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, log_beam_cut(options),
+                              stay, g->s_side), "beam_search");
+    HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_side));
+
+    launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->s_main),
+              "fwd_post_scan");
+    HIP_OK(hipEventRecord(g->ev[EV_FWD_END], g->s_main));
+
+    HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_BEAM_END], 0));
+    HIP_OK(hipEventRecord(g->ev[EV_SEQ_START], g->s_main));
+    launch_ok(ofk_sequence(g->pub.post_NTC, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data,
+                           g->pub.base_probs, g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N,
+                           state_len, phred_for(g, options), g->s_main), "sequence");
+    HIP_OK(hipEventRecord(g->ev[EV_SEQ_END], g->s_main));
+
+    fetch_outputs(g, T, N, moves, sequence, qstring);
+    g->timed = 1;
+}
+
+int openfish_amd_last_timings(const openfish_gpubuf_t *gpubuf, float *ms, int n) {
+    ofa_gpubuf_t *g = (ofa_gpubuf_t *)gpubuf;
+    if (!g || g->magic != OFA_MAGIC) die("gpubuf was not created by openfish_gpubuf_init");
+    if (!g->timed || !ms || n < 1) return 0;
+    HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_BWD], g->ev[EV_START], g->ev[EV_BWD_END]));
+    HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_FWD], g->ev[EV_BWD_END], g->ev[EV_FWD_END]));
+    HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_BEAM], g->ev[EV_BEAM_START], g->ev[EV_BEAM_END]));
+    HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_SEQ], g->ev[EV_SEQ_START], g->ev[EV_SEQ_END]));
+    HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_TOTAL], g->ev[EV_START], g->ev[EV_SEQ_END]));
+    if (n > OPENFISH_AMD_STAGE_COUNT) n = OPENFISH_AMD_STAGE_COUNT;
+    memcpy(ms, g->ms, sizeof(float) * (size_t)n);
+    return n;
+}
+
+/* ---- stages ---------------------------------------------------------------- */
+
+void openfish_amd_bwd_scan(int T, int N, int C, const void *scores, int state_len, float stay_score, float *bwd) {
+    openfish_opt_t o = DECODER_INIT;
+    check_scores(T, N, C, scores, state_len, &o);
+    launch_ok(ofk_bwd_scan(scores, bwd, T, N, state_len, stay_score, NULL), "bwd_scan");
+    HIP_OK(hipStreamSynchronize(0));
+}
+
+void openfish_amd_fwd_post_scan(int T, int N, int C, const void *scores, int state_len, float stay_score,
+                                const float *bwd, float *post) {
+    openfish_opt_t o = DECODER_INIT;
+    check_scores(T, N, C, scores, state_len, &o);
+    launch_ok(ofk_fwd_post_scan(scores, bwd, post, T, N, state_len, stay_score, NULL), "fwd_post_scan");
+    HIP_OK(hipStreamSynchronize(0));
+}
+
+void openfish_amd_beam_search(int T, int N, int C, const void *scores, int state_len,
+                              const openfish_opt_t *options, const float *bwd, const openfish_gpubuf_t *gpubuf) {
+    check_scores(T, N, C, scores, state_len, options);
+    ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
+    launch_ok(ofk_beam_search(scores, bwd, (ofk_beam_slot_t *)g->pub.beam_vector, (int32_t *)g->pub.states,
+                              g->pub.moves, T, N, state_len, log_beam_cut(options), options->blank_score, NULL),
+              "beam_search");
+    HIP_OK(hipStreamSynchronize(0));
+}
+
+void openfish_amd_sequence(int T, int N, int state_len, const openfish_opt_t *options, const float *post,
+                           const openfish_gpubuf_t *gpubuf) {
+    if (!options) die("options is NULL");
+    ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
+    launch_ok(ofk_sequence(post, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data, g->pub.base_probs,
+                           g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N, state_len,
+                           phred_for(g, options), NULL), "sequence");
+    HIP_OK(hipStreamSynchronize(0));
+}
+
+void openfish_amd_decode_from_tensors(int T, int N, int C, const void *scores, int state_len,
+                                      const openfish_opt_t *options, const float *bwd, const float *post,
+                                      const openfish_gpubuf_t *gpubuf, uint8_t **moves, char **sequence,
+                                      char **qstring) {
+    check_scores(T, N, C, scores, state_len, options);
+    ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
+    join_null_stream(g);
+    launch_ok(ofk_beam_search(scores, bwd, (ofk_beam_slot_t *)g->pub.beam_vector, (int32_t *)g->pub.states,
+                              g->pub.moves, T, N, state_len, log_beam_cut(options), options->blank_score,
+                              g->s_main), "beam_search");
+    launch_ok(ofk_sequence(post, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data, g->pub.base_probs,
+                           g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N, state_len,
+                           phred_for(g, options), g->s_main), "sequence");
+    fetch_outputs(g, T, N, moves, sequence, qstring);
+}
+
+/* ---- rotary embedding ------------------------------------------------------ */
+
+void openfish_rotary_emb_gpu(void *x_gpu, void *sin_gpu, void *cos_gpu, int batch_size, int seqlen, int nheads,
+                             int head_dim, int rotary_half, int stride_batch, int stride_seq, int stride_head) {
+    (void)head_dim; /* unused by the reference as well (src/rotary_emb_hip.h:36-45) */
+    launch_ok(ofk_rotary_emb(x_gpu, (const float *)sin_gpu, (const float *)cos_gpu, batch_size, seqlen, nheads,
+                             rotary_half, stride_batch, stride_seq, stride_head, NULL), "rotary_emb");
+    HIP_OK(hipStreamSynchronize(0));
+}
+
+/* ---- CPU entry points of the reference API: not carried by this library ---- */
+
+void openfish_decode_cpu(const int T, const int N, const int C, int nthreads, void *scores_TNC,
+                         const int state_len, const openfish_opt_t *options, uint8_t **moves, char **sequence,
+                         char **qstring) {
+    (void)T; (void)N; (void)C; (void)nthreads; (void)scores_TNC; (void)state_len; (void)options;
+    (void)moves; (void)sequence; (void)qstring;
+    die("openfish_decode_cpu: this library carries the GPU path only");
+}
+
+void openfish_rotary_emb_cpu(void *x, void *sin_buf, void *cos_buf, int batch_size, int seqlen, int nheads,
+                             int head_dim, int rotary_half, int stride_batch, int stride_seq, int stride_head,
+                             int nthreads) {
+    (void)x; (void)sin_buf; (void)cos_buf; (void)batch_size; (void)seqlen; (void)nheads; (void)head_dim;
+    (void)rotary_half; (void)stride_batch; (void)stride_seq; (void)stride_head; (void)nthreads;
+    die("openfish_rotary_emb_cpu: this library carries the GPU path only");
+}
+
+/* ---- device helpers -------------------------------------------------------- */
+
+void set_device_hip(int device) { HIP_OK(hipSetDevice(device)); }
+
+void *upload_scores_to_hip(const int T, const int N, const int C, const void *scores_TNC) {
+    void *dev = NULL;
+    const size_t bytes = 2 * (size_t)T * (size_t)N * (size_t)C;
+    HIP_OK(hipMalloc(&dev, bytes));
+    HIP_OK(hipMemcpy(dev, scores_TNC, bytes, hipMemcpyHostToDevice));
+    return dev;
+}
+
+void free_scores_hip(void *scores_TNC_gpu) { HIP_OK(hipFree(scores_TNC_gpu)); }
+
+static void dump_blob(const char *name, const void *dev, size_t bytes) {
+    void *host = host_alloc(bytes);
+    HIP_OK(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost));
+    FILE *fp = fopen(name, "w");
+    if (!fp || fwrite(host, 1, bytes, fp) != bytes) {
+        fprintf(stderr, "openfish: error writing %s: %s\n", name, strerror(errno));
+        exit(EXIT_FAILURE);
+    }
+    fclose(fp);
+    free(host);
+}
+
+void write_gpubuf_hip(const uint64_t T, const uint64_t N, const int state_len, const openfish_gpubuf_t *gpubuf) {
+    check_state_len(state_len);
+    const size_t S = (size_t)states_of(state_len), tens = sizeof(float) * N * (T + 1) * S, nt = N * T;
+    dump_blob("bwd_NTC.blob", gpubuf->bwd_NTC, tens);
+    dump_blob("post_NTC.blob", gpubuf->post_NTC, tens);
+    dump_blob("qual_data.blob", gpubuf->qual_data, sizeof(float) * 4 * nt);
+    dump_blob("base_probs.blob", gpubuf->base_probs, sizeof(float) * nt);
+    dump_blob("total_probs.blob", gpubuf->total_probs, sizeof(float) * nt);
+}
+
+void *openfish_amd_malloc(size_t bytes) {
+    void *dev = NULL;
+    HIP_OK(hipMalloc(&dev, bytes ? bytes : 1));
+    return dev;
+}
+void openfish_amd_free(void *dev) { HIP_OK(hipFree(dev)); }
+void openfish_amd_memcpy_h2d(void *dev, const void *host, size_t bytes) { HIP_OK(hipMemcpy(dev, host, bytes, hipMemcpyHostToDevice)); }
+void openfish_amd_memcpy_d2h(void *host, const void *dev, size_t bytes) { HIP_OK(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost)); }
+void openfish_amd_memset(void *dev, int value, size_t bytes) { HIP_OK(hipMemset(dev, value, bytes)); }
+void openfish_amd_sync(void) { HIP_OK(hipDeviceSynchronize()); }
+
+int openfish_amd_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+void openfish_amd_set_debug_flags(int flags) { ofk_set_beam_flags(flags & 1); }
+
+void openfish_amd_set_scan_mode(int fast) { ofk_set_scan_fast(fast ? 1 : 0); }
+
+const char *openfish_amd_version(void) { return "openfish-amd gfx950"; }

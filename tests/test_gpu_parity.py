@@ -1,0 +1,265 @@
+"""Parity of the HIP path with the CPU oracle, through the C-ABI, on a real MI355X.
+
+Tolerances (the acceptance bar of this decoder):
+  * bwd and post tensors: |gpu - cpu| <= 1e-3 * |cpu| element-wise (for posteriors
+    below the smallest normal fp32 number an absolute 1.2e-38 applies instead);
+  * moves, sequence, qstring: identical bytes when the beam/sequence stage is fed
+    the CPU path's own bwd/post tensors.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from openfish_amd import synth
+from oracle import crf_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+CASES = sorted(os.path.basename(p)[:-4] for p in glob.glob(os.path.join(GOLDEN, "*.npz")))
+GPU_CASES = [c for c in CASES if not c.startswith(("sl1", "sl2"))]  # the kernels cover 64, 256, 1024 states
+RTOL = 1e-3
+POST_ATOL = 1.2e-38
+
+
+@pytest.fixture(scope="module")
+def api():
+    from openfish_amd import api as _api
+    if _api.device_count() < 1:
+        pytest.skip("no HIP device")
+    _api.set_scan_mode(False)
+    _api.set_debug_flags(0)
+    return _api
+
+
+def load(name):
+    z = np.load(os.path.join(GOLDEN, name + ".npz"))
+    bc, bl, qs, qc = [float(v) for v in z["opt"]]
+    return z, int(z["state_len"]), dict(beam_cut=bc, blank_score=bl, q_shift=qs, q_scale=qc)
+
+
+def close(a, b, atol=0.0):
+    a, b = a.astype(np.float64), b.astype(np.float64)
+    bad = np.abs(a - b) > RTOL * np.abs(b) + atol
+    assert not bad.any(), "%d of %d elements beyond 1e-3 relative, worst %.3e" % (
+        bad.sum(), bad.size, (np.abs(a - b) / np.maximum(np.abs(b), 1e-300)).max())
+
+
+def gpu_scans(api, s16, state_len, stay=2.0):
+    T, N, C = s16.shape
+    S = 4 ** state_len
+    sc = api.upload_scores_to_hip(s16)
+    bwd = api.DeviceBuffer(4 * N * (T + 1) * S)
+    post = api.DeviceBuffer(4 * N * (T + 1) * S)
+    bwd.fill(0xFF)
+    post.fill(0xFF)
+    api.openfish_amd_bwd_scan(T, N, C, sc, state_len, stay, bwd)
+    api.openfish_amd_fwd_post_scan(T, N, C, sc, state_len, stay, bwd, post)
+    return bwd.to_host(np.float32, (N, T + 1, S)), post.to_host(np.float32, (N, T + 1, S))
+
+
+def gpu_from_tensors(api, s16, state_len, opt_kw, bwd, post):
+    T, N, C = s16.shape
+    sc = api.upload_scores_to_hip(s16)
+    gb = api.GpuBuf(T, N, state_len)
+    rb, rp = api.DeviceBuffer.from_host(bwd), api.DeviceBuffer.from_host(post)
+    out = api.openfish_amd_decode_from_tensors(T, N, C, sc, state_len, api.DECODER_INIT(**opt_kw), rb, rp, gb)
+    return out, gb
+
+
+# ---- golden vectors written by the compiled reference ---------------------------
+
+@pytest.mark.parametrize("name", GPU_CASES)
+def test_scans_match_reference_golden(api, name):
+    z, sl, opt = load(name)
+    bwd, post = gpu_scans(api, z["scores"], sl)
+    close(bwd, z["bwd"])
+    close(post, z["post"], POST_ATOL)
+
+
+@pytest.mark.parametrize("name", GPU_CASES)
+def test_beam_stage_bit_exact_on_reference_tensors(api, name):
+    z, sl, opt = load(name)
+    (mv, sq, qs), gb = gpu_from_tensors(api, z["scores"], sl, opt, z["bwd"], z["post"])
+    assert np.array_equal(mv, z["moves"])
+    assert np.array_equal(sq, z["sequence"])
+    assert np.array_equal(qs, z["qstring"])
+    assert np.array_equal(gb.tensor("total_probs"), z["total_probs"]) or \
+        np.allclose(gb.tensor("total_probs"), z["total_probs"], rtol=3e-7)
+    np.testing.assert_allclose(gb.tensor("qual_data"), z["qual_data"], rtol=3e-7)  # pow: last bit of libm
+
+
+@pytest.mark.parametrize("name", GPU_CASES)
+def test_whole_decode_on_golden(api, name):
+    """openfish_decode_gpu end to end; with the CPU-faithful scan arithmetic the GPU's own
+    tensors lead to the same calls as the reference's"""
+    z, sl, opt = load(name)
+    s16 = z["scores"]
+    T, N, C = s16.shape
+    if opt["blank_score"] != 2.0:
+        pytest.skip("the CPU scans ignore blank_score, the GPU entry point does not (as in the reference)")
+    sc = api.upload_scores_to_hip(s16)
+    gb = api.GpuBuf(T, N, sl)
+    mv, sq, qs = api.openfish_decode_gpu(T, N, C, sc, sl, api.DECODER_INIT(**opt), gb)
+    assert np.array_equal(mv, z["moves"]) and np.array_equal(sq, z["sequence"]) and np.array_equal(qs, z["qstring"])
+    t = gb.timings()
+    assert set(t) == set(api.STAGES) and all(v > 0 for v in t.values())
+
+
+def test_reference_in_repo_fixture_end_to_end(api):
+    """the reference's own known-answer test (fast model, N=1, T=1666); its fp32 scores are
+    all exactly representable in fp16"""
+    sc32 = np.fromfile(os.path.join(GOLDEN, "ref_fixture_scores.blob"), np.float32).reshape(1666, 1, 256)
+    s16 = sc32.astype(np.float16)
+    assert np.array_equal(s16.astype(np.float32), sc32)
+    sc = api.upload_scores_to_hip(s16)
+    gb = api.GpuBuf(1666, 1, 3)
+    mv, sq, qs = api.openfish_decode_gpu(1666, 1, 256, sc, 3, api.DECODER_INIT(q_scale=0.97, q_shift=-1.8), gb)
+    for got, name in ((mv, "moves"), (sq, "sequence"), (qs, "qstring")):
+        want = np.fromfile(os.path.join(GOLDEN, "ref_fixture_%s.blob" % name), np.uint8).reshape(1, 1666)
+        assert np.array_equal(got, want), name
+
+
+# ---- seeded inputs against the oracle ----------------------------------------------
+
+SHAPES = [
+    # state_len, T, N, stress
+    (3, 1, 1, False), (3, 2, 3, False), (3, 7, 5, False), (3, 9, 4, True), (3, 333, 13, True),
+    (4, 1, 2, False), (4, 5, 1, False), (4, 257, 9, False), (4, 130, 6, True),
+    (5, 3, 1, False), (5, 61, 3, False), (5, 40, 2, True),
+]
+
+
+@pytest.mark.parametrize("state_len,T,N,stress", SHAPES)
+def test_stages_against_oracle(api, state_len, T, N, stress):
+    """ragged shapes: T below the prefetch depth, N not a multiple of the chunks a
+    workgroup holds, single chunks"""
+    scale = synth.stress_scale(N) if stress else None
+    s16 = synth.crf_scores(T, N, state_len, seed=1000 + 7 * T + N, chunk_scale=scale)
+    kw = dict(q_scale=0.95, q_shift=-0.2)
+    ref = O.decode(s16.astype(np.float32), state_len, kw, nthreads=4)
+    bwd, post = gpu_scans(api, s16, state_len)
+    close(bwd, ref["bwd"])
+    close(post, ref["post"], POST_ATOL)
+    assert np.all(bwd[:, T, :] == 0.0)
+    (mv, sq, qs), gb = gpu_from_tensors(api, s16, state_len, kw, ref["bwd"], ref["post"])
+    assert np.array_equal(mv, ref["moves"])
+    assert np.array_equal(gb.tensor("states"), ref["states"])
+    assert np.array_equal(sq, ref["sequence"])
+    assert np.array_equal(qs, ref["qstring"])
+
+
+def test_fast_scan_mode_stays_within_two_ulp_of_bwd(api):
+    s16 = synth.crf_scores(400, 6, 4, seed=77)
+    ref = O.scans(s16.astype(np.float32), 4)
+    api.set_scan_mode(True)
+    try:
+        bwd, post = gpu_scans(api, s16, 4)
+    finally:
+        api.set_scan_mode(False)
+    np.testing.assert_allclose(bwd, ref[0], rtol=3e-7)
+    np.testing.assert_allclose(post, ref[2], rtol=5e-3, atol=POST_ATOL)
+
+
+def test_serial_merge_route_gives_identical_output(api):
+    """the route taken after a CRC collision (serial replay of the merges) must agree with
+    the parallel one whenever there is no collision"""
+    s16 = synth.crf_scores(300, 9, 4, seed=31, chunk_scale=synth.stress_scale(9))
+    kw = dict(q_scale=0.95, q_shift=-0.2)
+    ref = O.decode(s16.astype(np.float32), 4, kw, nthreads=4)
+    api.set_debug_flags(1)
+    try:
+        (mv, sq, qs), _ = gpu_from_tensors(api, s16, 4, kw, ref["bwd"], ref["post"])
+    finally:
+        api.set_debug_flags(0)
+    assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
+
+
+def test_options_beam_cut_and_blank_score(api):
+    s16 = synth.crf_scores(250, 5, 3, seed=41)
+    for kw in (dict(beam_cut=3.0), dict(beam_cut=1e6, blank_score=0.5), dict(beam_cut=0.0), dict(q_scale=1.3, q_shift=4.0)):
+        ref = O.decode(s16.astype(np.float32), 3, kw, nthreads=4)
+        (mv, sq, qs), _ = gpu_from_tensors(api, s16, 3, kw, ref["bwd"], ref["post"])
+        assert np.array_equal(mv, ref["moves"]), kw
+        assert np.array_equal(sq, ref["sequence"]), kw
+        assert np.array_equal(qs, ref["qstring"]), kw
+
+
+def test_gpubuf_is_reusable_for_smaller_batches(api):
+    gb = api.GpuBuf(200, 8, 3)
+    for T, N, seed in ((200, 8, 1), (77, 3, 2), (200, 8, 1)):
+        s16 = synth.crf_scores(T, N, 3, seed=seed)
+        ref = O.decode(s16.astype(np.float32), 3, nthreads=4)
+        sc = api.upload_scores_to_hip(s16)
+        mv, sq, qs = api.openfish_decode_gpu(T, N, 4 * 64, sc, 3, api.DECODER_INIT(), gb)
+        assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
+
+
+def test_constant_scores_closed_form(api):
+    T, N, sl, c = 64, 3, 3, 0.75
+    S = 4 ** sl
+    s16 = np.full((T, N, 4 * S), c, np.float16)
+    bwd, post = gpu_scans(api, s16, sl)
+    per_step = np.log(np.exp(2.0) + 4 * np.exp(c))
+    want = (T - np.arange(T + 1)) * per_step
+    np.testing.assert_allclose(bwd, np.broadcast_to(want[None, :, None], bwd.shape), rtol=2e-6)
+    np.testing.assert_allclose(post, 1.0 / S, rtol=1e-5)
+
+
+# ---- full benchmark sizes: properties + oracle on a slice of the chunks ------------
+
+FULL = [("fast", 3, 1666, 512, False, 16), ("hac", 4, 1666, 512, False, 12),
+        ("sup", 5, 1666, 256, False, 4), ("hac_stress", 4, 1666, 1024, True, 12)]
+
+
+@pytest.mark.parametrize("name,state_len,T,N,stress,sub", FULL)
+def test_full_size_configurations(api, name, state_len, T, N, stress, sub):
+    S, C = 4 ** state_len, 4 * 4 ** state_len
+    scale = synth.stress_scale(N) if stress else None
+    s16 = synth.crf_scores(T, N, state_len, seed=2025, chunk_scale=scale, threads=16)
+    kw = dict(q_scale=0.95, q_shift=-0.2)
+    sc = api.upload_scores_to_hip(s16)
+    gb = api.GpuBuf(T, N, state_len)
+    mv, sq, qs = api.openfish_decode_gpu(T, N, C, sc, state_len, api.DECODER_INIT(**kw), gb)
+
+    # size-independent properties of every chunk
+    assert mv.shape == (N, T) and set(np.unique(mv)) <= {0, 1} and np.all(mv[:, 0] == 1)
+    lens = mv.sum(axis=1)
+    pos = np.arange(T)[None, :]
+    inside = pos < lens[:, None]
+    assert np.all(np.isin(sq[inside], np.frombuffer(b"ACGT", np.uint8))) and np.all(sq[~inside] == 0)
+    assert np.all((qs[inside] >= 34) & (qs[inside] <= 83)) and np.all(qs[~inside] == 0)
+    for n in (0, N // 2, N - 1):  # the big tensors one chunk at a time
+        post = gb.tensor("post_NTC")[n]
+        np.testing.assert_allclose(post.sum(axis=1), 1.0, rtol=2e-5)
+        assert np.all(gb.tensor("bwd_NTC")[n][T] == 0.0)
+
+    # the oracle on the first `sub` chunks (chunks are independent)
+    ref = O.decode(np.ascontiguousarray(s16[:, :sub, :]).astype(np.float32), state_len, kw, nthreads=16)
+    close(gb.tensor("bwd_NTC")[:sub], ref["bwd"])
+    close(gb.tensor("post_NTC")[:sub], ref["post"], POST_ATOL)
+    s_sub = np.ascontiguousarray(s16[:, :sub, :])
+    (mv2, sq2, qs2), _ = gpu_from_tensors(api, s_sub, state_len, kw, ref["bwd"], ref["post"])
+    assert np.array_equal(mv2, ref["moves"]) and np.array_equal(sq2, ref["sequence"]) and np.array_equal(qs2, ref["qstring"])
+
+
+# ---- rotary embedding ------------------------------------------------------------------
+
+@pytest.mark.parametrize("batch,seqlen,nheads,head_dim,half", [(3, 17, 4, 16, 8), (2, 33, 8, 64, 32),
+                                                                (2, 5, 3, 10, 3), (1, 1, 1, 2, 1),
+                                                                (16, 833, 8, 64, 32)])
+def test_rotary_matches_cpu_path_rounded_to_half(api, batch, seqlen, nheads, head_dim, half):
+    rng = np.random.default_rng(batch * 100 + seqlen)
+    x16 = rng.standard_normal((batch, seqlen, nheads, head_dim)).astype(np.float16)
+    sn, cs = synth.rotary_tables(seqlen, half)
+    strides = (seqlen * nheads * head_dim, nheads * head_dim, head_dim)
+    want = O.rotary_emb(x16.astype(np.float32), sn, cs, batch, seqlen, nheads, head_dim, half, *strides)
+    want16 = want.reshape(x16.shape).astype(np.float16)
+    xd = api.DeviceBuffer.from_host(x16)
+    sd, cd = api.DeviceBuffer.from_host(sn), api.DeviceBuffer.from_host(cs)
+    api.openfish_rotary_emb_gpu(xd, sd, cd, batch, seqlen, nheads, head_dim, half, *strides)
+    got = xd.to_host(np.float16, x16.shape)
+    assert np.array_equal(got.view(np.uint16), want16.view(np.uint16))
+    assert np.array_equal(got[..., 2 * half:], x16[..., 2 * half:])  # beyond the rotary span: untouched
