@@ -27,7 +27,7 @@ C_OBJ   := $(BUILD)/openfish_host.o
 
 all: lib/libopenfish.a openfish_amd/libopenfish_amd.so
 
-$(BUILD)/%.o: $(SRC)/%.hip $(SRC)/kernels.h
+$(BUILD)/%.o: $(SRC)/%.hip $(SRC)/kernels.h $(SRC)/dmath.h
 	@mkdir -p $(BUILD)
 	$(HIPCC) $(HIPFLAGS) -c $< -o $@
 

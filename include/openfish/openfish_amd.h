@@ -122,6 +122,13 @@ void openfish_amd_set_debug_flags(int flags);
 void openfish_amd_set_scan_mode(int fast);
 
 /*
+ * Tuning knob of the scans: how many of the 4^state_len states one lane carries (4, 2
+ * or 1).  0, the default, picks the largest value that still gives every SIMD of the
+ * device a wavefront for the batch at hand.  Results do not depend on it.  Process-wide.
+ */
+void openfish_amd_set_scan_states_per_lane(int spl);
+
+/*
  * The 49 miss-probability thresholds behind the phred characters for one
  * (q_scale, q_shift): char(x) = 83 - #{j : x >= thr[j]} equals
  * (char)(33.5f + clamp(-10*log10f(x)*q_scale + q_shift, 1, 50)) of the reference

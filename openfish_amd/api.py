@@ -80,6 +80,7 @@ _SIGS = {
     "openfish_amd_last_timings": (_i, [_bufp, C.POINTER(C.c_float), _i]),
     "openfish_amd_set_debug_flags": (None, [_i]),
     "openfish_amd_set_scan_mode": (None, [_i]),
+    "openfish_amd_set_scan_states_per_lane": (None, [_i]),
     "openfish_amd_phred_table": (None, [_f, _f, C.POINTER(C.c_float)]),
     "openfish_amd_version": (C.c_char_p, []),
 }
@@ -244,6 +245,10 @@ def phred_table(q_scale, q_shift):
 
 def set_scan_mode(fast):
     _L.openfish_amd_set_scan_mode(1 if fast else 0)
+
+
+def set_scan_states_per_lane(spl):
+    _L.openfish_amd_set_scan_states_per_lane(int(spl))
 
 
 def set_debug_flags(flags):

@@ -1,0 +1,128 @@
+// Double-precision exp and log for the scans, written for the narrow domains the
+// scans need so that they cost a few dozen full-rate fp64 FMAs instead of a
+// general libm call:
+//   exp_nonpos(d) : e^d for a float d <= 0, relative error below 2^-46
+//   log_1to5(s)   : ln(s) for a float s in [1, 5] (a sum of five terms <= 1, one of
+//                   which is exactly 1), relative error below 2^-51
+// The CPU path evaluates exp and log in double and then rounds to fp32 (reference
+// src/decode_cpu.c:45-49); these stand in for its libm calls.  With the errors above
+// a result can round to a different fp32 value only when the exact value lies
+// within 2^-46 (relative) of a rounding boundary.
+//
+// The functions compile for host and device; the host build is what the accuracy
+// test links.
+#ifndef OPENFISH_AMD_DMATH_H
+#define OPENFISH_AMD_DMATH_H
+
+#include <stdint.h>
+#include <string.h>
+
+#if defined(__HIPCC__)
+#define OFA_HD __host__ __device__ __forceinline__
+#else
+#define OFA_HD static inline
+#endif
+
+namespace ofa {
+
+OFA_HD uint64_t bits_of(double x) {
+    uint64_t u;
+    memcpy(&u, &x, sizeof u);
+    return u;
+}
+OFA_HD double double_of(uint64_t u) {
+    double x;
+    memcpy(&x, &u, sizeof x);
+    return x;
+}
+OFA_HD uint32_t bits_of(float x) {
+    uint32_t u;
+    memcpy(&u, &x, sizeof u);
+    return u;
+}
+OFA_HD float float_of(uint32_t u) {
+    float x;
+    memcpy(&x, &u, sizeof x);
+    return x;
+}
+
+// e^d, d <= 0.  Arguments below -80 are treated as -80: e^-80 = 1.8e-35 is far below
+// half an ulp of the sum it is added to (the sum contains a term equal to 1), and as a
+// first term it rounds to an fp32 value that the later 1 absorbs just the same.
+OFA_HD double exp_nonpos(float d) {
+    const double x = (double)(d > -80.0f ? d : -80.0f);
+    const double kShift = 6755399441055744.0;  // 1.5 * 2^52: adding it rounds to an integer
+    const double kLog2e = 1.4426950408889634074;
+    const double kLn2Hi = 6.93147180369123816490e-01;  // 32 significant bits: n * kLn2Hi is exact
+    const double kLn2Lo = 1.90821492927058770002e-10;
+    const double t = __builtin_fma(x, kLog2e, kShift);
+    const double n = t - kShift;
+    double r = __builtin_fma(n, -kLn2Hi, x);
+    r = __builtin_fma(n, -kLn2Lo, r);  // |r| <= ln2/2
+    // Taylor series to degree 11: the remainder r^12/12! is below 2^-47
+    double p = 1.0 / 39916800.0;
+    p = __builtin_fma(p, r, 1.0 / 3628800.0);
+    p = __builtin_fma(p, r, 1.0 / 362880.0);
+    p = __builtin_fma(p, r, 1.0 / 40320.0);
+    p = __builtin_fma(p, r, 1.0 / 5040.0);
+    p = __builtin_fma(p, r, 1.0 / 720.0);
+    p = __builtin_fma(p, r, 1.0 / 120.0);
+    p = __builtin_fma(p, r, 1.0 / 24.0);
+    p = __builtin_fma(p, r, 1.0 / 6.0);
+    p = __builtin_fma(p, r, 0.5);
+    p = __builtin_fma(p, r, 1.0);
+    p = __builtin_fma(p, r, 1.0);
+    // p in [0.70, 1.42]; n >= -116: scaling by 2^n is an add to the exponent field
+    const uint64_t scaled = bits_of(p) + ((uint64_t)(int64_t)(int32_t)(uint32_t)bits_of(t) << 52);
+    return double_of(scaled);
+}
+
+// ln(s) for a float s in [1, 5].  s = 2^k * u with u in [sqrt(1/2), sqrt(2)),
+// ln(u) = 2 atanh(z), z = (u - 1) / (u + 1), |z| <= 0.1716.
+OFA_HD double log_1to5(float s) {
+    const uint32_t b = bits_of(s);
+    const uint32_t frac = b & 0x007fffffu;
+    const uint32_t up = frac > 0x003504f3u ? 1u : 0u;  // mantissa above sqrt(2): use u/2, k+1
+    const int k = (int)(b >> 23) - 127 + (int)up;
+    const float u = float_of(frac | ((127u - up) << 23));
+    const double f = (double)u - 1.0;  // exact
+    const double den = 2.0 + f;        // exact
+#if defined(__HIP_DEVICE_COMPILE__)
+    double y = (double)__builtin_amdgcn_rcpf((float)den);
+#else
+    double y = (double)(1.0f / (float)den);
+#endif
+    y = __builtin_fma(__builtin_fma(-den, y, 1.0), y, y);  // Newton: 2^-22 -> 2^-44
+    y = __builtin_fma(__builtin_fma(-den, y, 1.0), y, y);  // -> full double
+    double z = f * y;
+    z = __builtin_fma(__builtin_fma(-z, den, f), y, z);    // residual correction of the quotient
+    const double w = z * z;  // <= 0.02944; the series is cut after w^9/21 < 2^-55
+    double p = 1.0 / 19.0;
+    p = __builtin_fma(p, w, 1.0 / 17.0);
+    p = __builtin_fma(p, w, 1.0 / 15.0);
+    p = __builtin_fma(p, w, 1.0 / 13.0);
+    p = __builtin_fma(p, w, 1.0 / 11.0);
+    p = __builtin_fma(p, w, 1.0 / 9.0);
+    p = __builtin_fma(p, w, 1.0 / 7.0);
+    p = __builtin_fma(p, w, 1.0 / 5.0);
+    p = __builtin_fma(p, w, 1.0 / 3.0);
+    const double z2 = z + z;
+    const double lu = __builtin_fma(z2 * w, p, z2);
+    const double kLn2 = 0.69314718055994530942;
+    return __builtin_fma((double)k, kLn2, lu);
+}
+
+// max + ln(sum_i e^(v_i - max)) with the CPU path's roundings: fp32 differences, the
+// running sum rounded to fp32 after every term, one rounding of the final sum.
+OFA_HD float lse5_cpu_rounding(float v0, float v1, float v2, float v3, float v4, float m) {
+    float s = (float)exp_nonpos(v0 - m);
+    s = (float)((double)s + exp_nonpos(v1 - m));
+    s = (float)((double)s + exp_nonpos(v2 - m));
+    s = (float)((double)s + exp_nonpos(v3 - m));
+    s = (float)((double)s + exp_nonpos(v4 - m));
+    return (float)((double)m + log_1to5(s));
+}
+
+}  // namespace ofa
+
+#endif

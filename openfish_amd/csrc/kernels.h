@@ -22,6 +22,8 @@ typedef uint16_t ofk_beam_slot_t;
 /* 0 (default): scans reproduce the CPU path's double exp/log and fp32 roundings;
  * 1: scans use the hardware fp32 exp/log (faster, last-bit differences). */
 void ofk_set_scan_fast(int on);
+/* states per lane of the scans: 4, 2 or 1; 0 (default) chooses from the batch size */
+void ofk_set_scan_states_per_lane(int spl);
 int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, float stay,
                  void *stream);
 int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N,

@@ -457,4 +457,6 @@ void openfish_amd_set_debug_flags(int flags) { ofk_set_beam_flags(flags & 1); }
 
 void openfish_amd_set_scan_mode(int fast) { ofk_set_scan_fast(fast ? 1 : 0); }
 
+void openfish_amd_set_scan_states_per_lane(int spl) { ofk_set_scan_states_per_lane(spl); }
+
 const char *openfish_amd_version(void) { return "openfish-amd gfx950"; }
