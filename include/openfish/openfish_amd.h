@@ -136,6 +136,14 @@ void openfish_amd_set_scan_states_per_lane(int spl);
  */
 void openfish_amd_phred_table(float q_scale, float q_shift, float *thr49);
 
+/*
+ * The table behind log(1 + e^-gap), gap in [0, 17), that the beam search uses when it
+ * folds a stay into a step (reference log_sum_exp, src/beam_search.c:43-47): 68 cells of
+ * width 1/4, each 9 coefficients (lowest degree first) of a polynomial in
+ * s = 8 * (gap - cell centre).  Writes 612 doubles.  Host-only; needs no device.
+ */
+void openfish_amd_lse_table(double *out);
+
 /* library build tag, e.g. "openfish-amd gfx950" */
 const char *openfish_amd_version(void);
 

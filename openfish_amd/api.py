@@ -81,6 +81,7 @@ _SIGS = {
     "openfish_amd_set_debug_flags": (None, [_i]),
     "openfish_amd_set_scan_mode": (None, [_i]),
     "openfish_amd_set_scan_states_per_lane": (None, [_i]),
+    "openfish_amd_lse_table": (None, [C.POINTER(C.c_double)]),
     "openfish_amd_phred_table": (None, [_f, _f, C.POINTER(C.c_float)]),
     "openfish_amd_version": (C.c_char_p, []),
 }
@@ -241,6 +242,13 @@ def phred_table(q_scale, q_shift):
     thr = (C.c_float * 49)()
     _L.openfish_amd_phred_table(q_scale, q_shift, thr)
     return np.array(thr[:], dtype=np.float32)
+
+
+def lse_table():
+    """[68][9] coefficients of log(1 + e^-gap) per quarter-unit cell"""
+    tab = (C.c_double * (68 * 9))()
+    _L.openfish_amd_lse_table(tab)
+    return np.array(tab[:], dtype=np.float64).reshape(68, 9)
 
 
 def set_scan_mode(fast):

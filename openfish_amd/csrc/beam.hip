@@ -114,11 +114,20 @@ __device__ __forceinline__ int observe(int *flag) {
 }
 
 // log(e^x + e^y) with the correction evaluated in double and dropped for gaps >= 17
-// (reference src/beam_search.c:43-47)
-__device__ __forceinline__ float log_sum_exp(float x, float y) {
+// (reference src/beam_search.c:43-47).  The correction log(1 + e^-gap) comes from a
+// piecewise polynomial kept in LDS: a handful of dependent FMAs instead of an exp
+// followed by a log, which matters because every merge sits on the search's serial path.
+__device__ __forceinline__ float log_sum_exp(float x, float y, const double *table) {
     const float gap = fabsf(x - y);
     const float top = x > y ? x : y;
-    const double corr = gap < 17.0f ? log(1.0 + exp(-(double)gap)) : 0.0;
+    int cell = (int)(gap * 4.0f);
+    cell = cell < OFK_LSE_CELLS - 1 ? cell : OFK_LSE_CELLS - 1;
+    const double *c = table + cell * OFK_LSE_COEFS;
+    const double s = ((double)gap - (0.25 * cell + 0.125)) * 8.0;
+    double p = c[8];
+#pragma unroll
+    for (int k = 7; k >= 0; --k) p = __builtin_fma(p, s, c[k]);
+    const double corr = gap < 17.0f ? p : 0.0;
     return (float)((double)top + corr);
 }
 
@@ -157,6 +166,18 @@ struct RowRegs {
     }
 };
 
+#ifdef OFK_BEAM_PROFILE
+__device__ unsigned long long g_beam_prof[16];
+#define PROF_MARK(k)                                              \
+    do {                                                          \
+        const unsigned long long now_ = __builtin_amdgcn_s_memtime(); \
+        prof_[k] += now_ - last_;                                 \
+        last_ = now_;                                             \
+    } while (0)
+#else
+#define PROF_MARK(k) do { } while (0)
+#endif
+
 template <int S>
 struct BeamCfg {
     static constexpr int kBits = S == 64 ? 6 : S == 256 ? 8 : 10;
@@ -165,15 +186,29 @@ struct BeamCfg {
     static constexpr int kTraceBlock = 128;             // time steps staged per traceback block
 };
 
+// one beam element as handed from one time step to the next
+struct __attribute__((aligned(16))) Elem {
+    uint32_t hash;
+    float score;
+    uint32_t info;  // state | prev << 16 | stay << 21
+    uint32_t pad;
+};
+// mailbox of one step candidate (index 4i+b): its score, and the stay that claims it
+struct __attribute__((aligned(16))) SlotRec {
+    uint32_t tag;   // (t + 1) << 5 | stay element, written by the claiming stay at step t
+    float stay;     // that stay's score
+    float step;     // the step candidate's score, written by its own lane
+    uint32_t pad;
+};
+
 struct BeamShared {
-    uint32_t hash[kW];
-    int32_t state[kW];
-    float score[kW];
-    uint32_t meta[kW];       // prev | stay << 5
-    float cand[5 * kW];      // candidate scores: steps at 4i+b, stays at 128+i
-    uint8_t owner[4 * kW];   // which stay claimed a step during a merge
-    int ready;               // rows stored by the loader wave
-    int consumed;            // rows the search wave is done with
+    uint32_t hash[kW];     // hashes of the current beam, contiguous for the match sweep
+    Elem elem[kW];
+    SlotRec rec[4 * kW];
+    float stay_score[kW];  // only used by the serial replay of merges
+    double lse[OFK_LSE_DOUBLES];
+    int ready;             // rows stored by the loader wave
+    int consumed;          // rows the search wave is done with
 };
 
 template <int S>
@@ -181,7 +216,8 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
                                                    const float *__restrict__ bwd,
                                                    ofk_beam_slot_t *__restrict__ beam,
                                                    int32_t *__restrict__ states, uint8_t *__restrict__ moves,
-                                                   int T, int N, float log_cut, float stay, int flags) {
+                                                   int T, int N, float log_cut, float stay, int flags,
+                                                   const double *__restrict__ lse_table) {
     using Cfg = BeamCfg<S>;
     constexpr int BITS = Cfg::kBits;
     constexpr int LR = Cfg::kLdsRows;
@@ -276,10 +312,11 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
         const float thr = key_float(prefix);
         if (lane < kW) {
             sh.hash[lane] = 0;
-            sh.state[lane] = 0;
-            sh.score[lane] = 0.f;
-            sh.meta[lane] = 0;
+            sh.elem[lane] = Elem{0u, 0.f, 0u, 0u};
         }
+        sh.rec[lane].tag = 0;  // tags of real time steps start at 1 << 5
+        sh.rec[lane + 64].tag = 0;
+        for (int x = lane; x < OFK_LSE_DOUBLES; x += 64) sh.lse[x] = lse_table[x];
         wave_fence();
         int taken = 0;
 #pragma unroll
@@ -288,28 +325,51 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
             const uint64_t m = ballot(ok);
             const int rank = taken + popc64(m & (((uint64_t)1 << lane) - 1));
             if (ok && rank < kW) {
-                const int s = j * 64 + lane;
-                sh.hash[rank] = crc32_word(kSeed, (uint32_t)s);
-                sh.state[rank] = s;
+                const uint32_t s = (uint32_t)(j * 64 + lane);
+                const uint32_t hs = crc32_word(kSeed, s);
+                sh.hash[rank] = hs;
+                sh.elem[rank] = Elem{hs, 0.f, s, 0u};
             }
             taken += popc64(m);
         }
         wave_fence();
     }
-    uint32_t hash = sh.hash[i];
-    int state = sh.state[i];
-    float score = 0.f;
+    uint32_t hash, info;
+    float score;
+    {
+        const Elem e = sh.elem[i];
+        hash = e.hash;
+        score = e.score;
+        info = e.info;
+    }
+    int state = (int)(info & 0xFFFFu);
     int w = kW;
     ofk_beam_slot_t *bv = beam + (size_t)n * (size_t)(T + 1) * kW;
     if (lane < kW) bv[lane] = (ofk_beam_slot_t)state;
 
+#ifdef OFK_BEAM_PROFILE
+    unsigned long long prof_[16] = {0};
+    unsigned long long last_ = __builtin_amdgcn_s_memtime();
+#endif
+    // The search is a chain of dependent short instructions; when it shares a SIMD with
+    // throughput-bound waves (the forward scan runs at the same time) it should win the
+    // issue arbitration.
+    __builtin_amdgcn_s_setprio(3);
+    int rows_ready = 0;  // last value seen of the loader's counter; it is usually several rows ahead
     for (int t = 0; t < T; ++t) {
-        while (observe(&sh.ready) <= t) __builtin_amdgcn_s_sleep(1);
+        PROF_MARK(0);
+        while (rows_ready <= t) {
+            rows_ready = observe(&sh.ready);
+            if (rows_ready <= t) __builtin_amdgcn_s_sleep(1);
+        }
+        PROF_MARK(1);
         const int slot = t % LR;
         const _Float16 *rs = row_s[slot];
         const float *rb = row_b[slot];
 
         const bool valid = i < w;
+        const uint64_t vm = ballot(valid);          // live elements, both halves
+        const uint64_t vs = vm & 0xFFFFFFFFull;     // their stay candidates sit on lanes < 32
         const int lo4 = (state << 2) & (S - 1);
         const int top = state >> (BITS - 2);
         const int b0 = 2 * h;
@@ -322,7 +382,11 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
         float cs = (score + stay) + gst;
         const uint32_t h0 = crc2(hash, (uint32_t)b0);
         const uint32_t h1 = crc2(hash, (uint32_t)b0 + 1u);
+        SlotRec *my_rec = &sh.rec[4 * i + b0];
+        my_rec[0].step = c0;
+        my_rec[1].step = c1;
 
+        PROF_MARK(2);
         // which previous element j has hash_j == crc^-1(hash_i, last base of i)
         uint32_t match;
         {
@@ -343,74 +407,89 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
             match = valid ? (m & live) : 0u;
         }
 
-        if (ballot(match != 0) != 0) {
-            // merge stays with the step spelling the same sequence (src/beam_search.c:281-316)
-            sh.cand[4 * i + b0] = c0;
-            sh.cand[4 * i + b0 + 1] = c1;
-            const bool mine = h == 0 && match != 0;
-            const int j = __builtin_ctz(match | 0x80000000u);
-            const int target = 4 * (j & 31) + (state & 3);
-            if (h == 0) sh.cand[4 * kW + i] = cs;
-            if (mine) sh.owner[target] = (uint8_t)i;
+        PROF_MARK(3);
+        // merge stays with the step spelling the same sequence (src/beam_search.c:281-316).
+        // The stay posts its score into the mailbox of the step it matches; then both
+        // sides read each other's score and apply their half of the merge.
+        const bool mine = h == 0 && match != 0;
+        if (ballot(mine) != 0) {
+            const uint32_t now = (uint32_t)(t + 1);
+            const uint32_t mytag = (now << 5) | (uint32_t)i;
+            const int target = 4 * (__builtin_ctz(match | 0x80000000u) & 31) + (state & 3);
+            if (mine) *reinterpret_cast<uint2 *>(&sh.rec[target]) = make_uint2(mytag, __float_as_uint(cs));
             wave_fence();
-            bool odd = false;
-            float other = 0.f;
-            if (mine) {
-                other = sh.cand[target];
-                odd = (match & (match - 1)) != 0 || sh.owner[target] != (uint8_t)i;
-            }
+            const uint4 claimed = mine ? *reinterpret_cast<const uint4 *>(&sh.rec[target]) : make_uint4(0, 0, 0, 0);
+            const uint4 box0 = *reinterpret_cast<const uint4 *>(&my_rec[0]);
+            const uint4 box1 = *reinterpret_cast<const uint4 *>(&my_rec[1]);
+            const bool odd = mine && ((match & (match - 1)) != 0 || claimed.x != mytag);
             if (ballot(odd) != 0 || (flags & 1)) {
                 // A stay with several equal hashes, or a step claimed by two stays (only
                 // possible after a CRC collision): replay the merges one by one in the
                 // CPU path's order.
+                if (h == 0) sh.stay_score[i] = cs;
                 wave_fence();
                 if (lane == 0) {
                     for (int a = 0; a < w; ++a) {
                         const uint32_t ha = sh.hash[a];
-                        const int base = sh.state[a] & 3;
-                        const int si = 4 * kW + a;
+                        const uint32_t base = sh.elem[a].info & 3u;
                         for (int b = 0; b < w; ++b) {
-                            if (crc2(sh.hash[b], (uint32_t)base) != ha) continue;
-                            const int st = 4 * b + base;
-                            const float folded = log_sum_exp(sh.cand[si], sh.cand[st]);
-                            if (sh.cand[si] > sh.cand[st]) {
-                                sh.cand[si] = folded;
-                                sh.cand[st] = -FLT_MAX;
+                            if (crc2(sh.hash[b], base) != ha) continue;
+                            SlotRec *st = &sh.rec[4 * b + (int)base];
+                            const float folded = log_sum_exp(sh.stay_score[a], st->step, sh.lse);
+                            if (sh.stay_score[a] > st->step) {
+                                sh.stay_score[a] = folded;
+                                st->step = -FLT_MAX;
                             } else {
-                                sh.cand[st] = folded;
-                                sh.cand[si] = -FLT_MAX;
+                                st->step = folded;
+                                sh.stay_score[a] = -FLT_MAX;
                             }
                         }
                     }
                 }
                 wave_fence();
-                if (h == 0) cs = sh.cand[4 * kW + i];
+                if (h == 0) cs = sh.stay_score[i];
+                c0 = my_rec[0].step;
+                c1 = my_rec[1].step;
             } else {
+                // Of every matched pair exactly one side survives and needs the folded
+                // score; the other becomes -FLT_MAX.  A lane rarely has more than one fold
+                // to compute (its stay, or one of its two steps), so the folds are taken
+                // one per lane and round, all lanes evaluating the polynomial together.
+                const float other = __uint_as_float(claimed.z);
+                const float st0 = __uint_as_float(box0.y), st1 = __uint_as_float(box1.y);
+                const bool hit0 = (box0.x >> 5) == now, hit1 = (box1.x >> 5) == now;
+                unsigned pend = 0;
                 if (mine) {
-                    const float folded = log_sum_exp(cs, other);
-                    if (cs > other) {
-                        cs = folded;
-                        sh.cand[target] = -FLT_MAX;
-                    } else {
-                        cs = -FLT_MAX;
-                        sh.cand[target] = folded;
-                    }
+                    if (cs > other) pend |= 1u; else cs = -FLT_MAX;
                 }
-                wave_fence();
+                if (hit0) {
+                    if (st0 > c0) c0 = -FLT_MAX; else pend |= 2u;
+                }
+                if (hit1) {
+                    if (st1 > c1) c1 = -FLT_MAX; else pend |= 4u;
+                }
+                while (ballot(pend != 0) != 0) {
+                    const unsigned pick = pend & (0u - pend);
+                    const float x = pick == 1u ? cs : pick == 2u ? st0 : st1;
+                    const float y = pick == 1u ? other : pick == 2u ? c0 : c1;
+                    const float folded = log_sum_exp(x, y, sh.lse);
+                    if (pick == 1u) cs = folded;
+                    if (pick == 2u) c0 = folded;
+                    if (pick == 4u) c1 = folded;
+                    pend ^= pick;
+                }
             }
-            c0 = sh.cand[4 * i + b0];
-            c1 = sh.cand[4 * i + b0 + 1];
         }
 
+        PROF_MARK(4);
         // cut-off (src/beam_search.c:320-381)
-        const bool has_stay = valid && h == 0;
         float best = -FLT_MAX;
         if (valid) best = fmaxf(c0, c1);
-        if (has_stay) best = fmaxf(best, cs);
+        if (valid && h == 0) best = fmaxf(best, cs);
         best = wave_max(best);
 
         float cut = best - log_cut;
-        uint64_t k0 = ballot(valid && c0 >= cut), k1 = ballot(valid && c1 >= cut), ks = ballot(has_stay && cs >= cut);
+        uint64_t k0 = ballot(c0 >= cut) & vm, k1 = ballot(c1 >= cut) & vm, ks = ballot(cs >= cut) & vs;
         int kept = popc64(k0) + popc64(k1) + popc64(ks);
         if (kept > kW) {
             float lo = cut, hi = best;
@@ -423,22 +502,23 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
                     hi = cut;
                     cut = (cut + lo) / 2.0f;
                 }
-                k0 = ballot(valid && c0 >= cut);
-                k1 = ballot(valid && c1 >= cut);
-                ks = ballot(has_stay && cs >= cut);
+                k0 = ballot(c0 >= cut) & vm;
+                k1 = ballot(c1 >= cut) & vm;
+                ks = ballot(cs >= cut) & vs;
                 kept = popc64(k0) + popc64(k1) + popc64(ks);
                 ++guesses;
             }
             if (guesses == 10) {
                 cut = hi;
-                k0 = ballot(valid && c0 >= cut);
-                k1 = ballot(valid && c1 >= cut);
-                ks = ballot(has_stay && cs >= cut);
+                k0 = ballot(c0 >= cut) & vm;
+                k1 = ballot(c1 >= cut) & vm;
+                ks = ballot(cs >= cut) & vs;
                 kept = popc64(k0) + popc64(k1) + popc64(ks);
             }
             if (kept > kW) kept = kW;
         }
 
+        PROF_MARK(5);
         // survivors in candidate order: steps (i, b) by i then b, then stays by i
         {
             const int before = popc64(k0 & below) + popc64(k1 & below);
@@ -448,39 +528,34 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
             const int rank0 = before + same;
             const int rank1 = rank0 + (keep0 ? 1 : 0);
             const int ranks = popc64(k0) + popc64(k1) + popc64(ks & below);
-            wave_fence();
+            const uint32_t from = (uint32_t)i << 16;
             if (keep0 && rank0 < kW) {
                 sh.hash[rank0] = h0;
-                sh.state[rank0] = lo4 + b0;
-                sh.score[rank0] = c0;
-                sh.meta[rank0] = (uint32_t)i;
+                sh.elem[rank0] = Elem{h0, c0, (uint32_t)(lo4 + b0) | from, 0u};
             }
             if (keep1 && rank1 < kW) {
                 sh.hash[rank1] = h1;
-                sh.state[rank1] = lo4 + b0 + 1;
-                sh.score[rank1] = c1;
-                sh.meta[rank1] = (uint32_t)i;
+                sh.elem[rank1] = Elem{h1, c1, (uint32_t)(lo4 + b0 + 1) | from, 0u};
             }
             if (keeps && ranks < kW) {
                 sh.hash[ranks] = hash;
-                sh.state[ranks] = state;
-                sh.score[ranks] = cs;
-                sh.meta[ranks] = (uint32_t)i | 32u;
+                sh.elem[ranks] = Elem{hash, cs, (uint32_t)state | from | (1u << 21), 0u};
             }
             wave_fence();
         }
         w = kept;
-        uint32_t meta = 0;
         if (i < w) {
-            hash = sh.hash[i];
-            state = sh.state[i];
-            score = sh.score[i];
-            meta = sh.meta[i];
+            const Elem e = sh.elem[i];
+            hash = e.hash;
+            score = e.score;
+            info = e.info;
         } else {
-            state = 0;
             score = 0.f;
+            info = 0;
         }
+        state = (int)(info & 0xFFFFu);
 
+        PROF_MARK(6);
         // last block: the best survivor goes to slot 0 (src/beam_search.c:398-414)
         if (t == T - 1) {
             const bool in = i < w;
@@ -489,17 +564,11 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
             const int arg = (top_score > -FLT_MAX && at != 0) ? __builtin_ctzll(at) : 0;
             if (arg != 0) {
                 const uint32_t hash0 = lane_u(hash, 0), hasha = lane_u(hash, arg);
-                const int st0 = (int)lane_u((uint32_t)state, 0), sta = (int)lane_u((uint32_t)state, arg);
+                const uint32_t in0 = lane_u(info, 0), ina = lane_u(info, arg);
                 const float sc0 = lane_f(score, 0), sca = lane_f(score, arg);
-                const uint32_t me0 = lane_u(meta, 0), mea = lane_u(meta, arg);
-                if (i == 0) { hash = hasha; state = sta; score = sca; meta = mea; }
-                if (i == arg) { hash = hash0; state = st0; score = sc0; meta = me0; }
-                wave_fence();
-                if (lane == 0 || lane == arg) {
-                    sh.hash[i] = hash;
-                    sh.state[i] = state;
-                }
-                wave_fence();
+                if (i == 0) { hash = hasha; info = ina; score = sca; }
+                if (i == arg) { hash = hash0; info = in0; score = sc0; }
+                state = (int)(info & 0xFFFFu);
             }
         }
 
@@ -508,11 +577,13 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
             score = score - rb[state];
             if (h == 0)
                 bv[(size_t)(t + 1) * kW + i] =
-                    (ofk_beam_slot_t)((uint32_t)state | ((meta & 31u) << 10) | ((meta >> 5) << 15));
+                    (ofk_beam_slot_t)((uint32_t)state | (((info >> 16) & 31u) << 10) | (((info >> 21) & 1u) << 15));
         }
+        PROF_MARK(7);
         publish(&sh.consumed, t + 1);
     }
 
+    PROF_MARK(7);
     // ---- traceback from slot 0 of the last block (src/beam_search.c:432-439) ----
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -541,13 +612,19 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
         }
         wave_fence();
     }
+#ifdef OFK_BEAM_PROFILE
+    PROF_MARK(8);
+    if (blockIdx.x == 0 && lane == 0)
+        for (int k = 0; k < 16; ++k) g_beam_prof[k] = prof_[k];
+#endif
 }
 
 template <int S>
 int launch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
-                uint8_t *moves, int T, int N, float log_cut, float stay, int flags, hipStream_t st) {
+                uint8_t *moves, int T, int N, float log_cut, float stay, int flags, const double *lse_table,
+                hipStream_t st) {
     hipLaunchKernelGGL((beam_kernel<S>), dim3(N), dim3(128), 0, st, static_cast<const _Float16 *>(scores),
-                       bwd, beam, states, moves, T, N, log_cut, stay, flags);
+                       bwd, beam, states, moves, T, N, log_cut, stay, flags, lse_table);
     return (int)hipGetLastError();
 }
 
@@ -557,17 +634,23 @@ int g_beam_flags = 0;
 
 extern "C" void ofk_set_beam_flags(int flags) { g_beam_flags = flags; }
 
+#ifdef OFK_BEAM_PROFILE
+extern "C" void ofk_beam_profile(unsigned long long *out16) {
+    (void)hipMemcpyFromSymbol(out16, HIP_SYMBOL(g_beam_prof), sizeof(unsigned long long) * 16);
+}
+#endif
+
 extern "C" int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                                uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
-                               void *stream) {
-    if (!scores || !bwd || !beam || !states || !moves || T < 1 || N < 1) return OFK_BAD_ARGS;
+                               const double *lse_table, void *stream) {
+    if (!scores || !bwd || !beam || !states || !moves || !lse_table || T < 1 || N < 1) return OFK_BAD_ARGS;
     if ((reinterpret_cast<uintptr_t>(scores) | reinterpret_cast<uintptr_t>(bwd) | reinterpret_cast<uintptr_t>(beam)) & 15u)
         return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (state_len) {
-        case 3: return launch_beam<64>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, st);
-        case 4: return launch_beam<256>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, st);
-        case 5: return launch_beam<1024>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, st);
+        case 3: return launch_beam<64>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, lse_table, st);
+        case 4: return launch_beam<256>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, lse_table, st);
+        case 5: return launch_beam<1024>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, lse_table, st);
         default: return OFK_BAD_ARGS;
     }
 }

@@ -77,16 +77,10 @@ OFA_HD double exp_nonpos(float d) {
     return double_of(scaled);
 }
 
-// ln(s) for a float s in [1, 5].  s = 2^k * u with u in [sqrt(1/2), sqrt(2)),
-// ln(u) = 2 atanh(z), z = (u - 1) / (u + 1), |z| <= 0.1716.
-OFA_HD double log_1to5(float s) {
-    const uint32_t b = bits_of(s);
-    const uint32_t frac = b & 0x007fffffu;
-    const uint32_t up = frac > 0x003504f3u ? 1u : 0u;  // mantissa above sqrt(2): use u/2, k+1
-    const int k = (int)(b >> 23) - 127 + (int)up;
-    const float u = float_of(frac | ((127u - up) << 23));
-    const double f = (double)u - 1.0;  // exact
-    const double den = 2.0 + f;        // exact
+// k*ln2 + ln(1 + f) for f in [sqrt(1/2) - 1, sqrt(2) - 1]:
+// ln(1 + f) = 2 atanh(z), z = f / (2 + f), |z| <= 0.1716.
+OFA_HD double log_core(double f, int k) {
+    const double den = 2.0 + f;
 #if defined(__HIP_DEVICE_COMPILE__)
     double y = (double)__builtin_amdgcn_rcpf((float)den);
 #else
@@ -110,6 +104,25 @@ OFA_HD double log_1to5(float s) {
     const double lu = __builtin_fma(z2 * w, p, z2);
     const double kLn2 = 0.69314718055994530942;
     return __builtin_fma((double)k, kLn2, lu);
+}
+
+// ln(s) for a float s in [1, 5]: s = 2^k * u with u in [sqrt(1/2), sqrt(2))
+OFA_HD double log_1to5(float s) {
+    const uint32_t b = bits_of(s);
+    const uint32_t frac = b & 0x007fffffu;
+    const uint32_t up = frac > 0x003504f3u ? 1u : 0u;  // mantissa above sqrt(2): use u/2, k+1
+    const int k = (int)(b >> 23) - 127 + (int)up;
+    const float u = float_of(frac | ((127u - up) << 23));
+    return log_core((double)u - 1.0, k);  // the difference is exact
+}
+
+// ln(1 + e^-gap) for a float gap in [0, 17): the correction term of log(e^x + e^y)
+// (reference src/beam_search.c:43-47), absolute error below 2^-46
+OFA_HD double log1p_exp_neg(float gap) {
+    const double x = 1.0 + exp_nonpos(-gap);  // in (1, 2]
+    const bool up = x > 1.4142135623730951;
+    const double u = up ? 0.5 * x : x;
+    return log_core(u - 1.0, up ? 1 : 0);  // the difference is exact
 }
 
 // max + ln(sum_i e^(v_i - max)) with the CPU path's roundings: fp32 differences, the

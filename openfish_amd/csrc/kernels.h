@@ -28,9 +28,17 @@ int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, fl
                  void *stream);
 int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N,
                       int state_len, float stay, void *stream);
+/* Table behind log(1 + e^-gap), the correction of a pairwise log-sum-exp, for gap in
+ * [0, 17): OFK_LSE_CELLS cells of width 1/4, each a degree-8 polynomial in
+ * s = 8 * (gap - centre) in [-1, 1], coefficients lowest degree first.  Built on the
+ * host in long double (ofk_lse_table_build), absolute error below 2^-46. */
+#define OFK_LSE_CELLS 68
+#define OFK_LSE_COEFS 9
+#define OFK_LSE_DOUBLES (OFK_LSE_CELLS * OFK_LSE_COEFS)
+
 int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                     uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
-                    void *stream);
+                    const double *lse_table, void *stream);
 /* bit 0: replay every stay/step merge one by one in CPU order (the path otherwise taken
  * only after a hash collision); results must not change.  For tests. */
 void ofk_set_beam_flags(int flags);

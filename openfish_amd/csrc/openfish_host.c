@@ -78,6 +78,40 @@ static void *host_alloc(size_t bytes) {
     return p;
 }
 
+/* ---- table of log(1 + e^-gap) for the beam search's merges -------------------
+ *
+ * The CPU path folds two scores with log(1.0 + exp(-gap)) in double (reference
+ * src/beam_search.c:43-47).  On the device that value is read off a piecewise
+ * polynomial: per cell of width 1/4 the degree-8 interpolant through the Chebyshev
+ * nodes, fitted here in long double.  The interpolation error is below 1e-15, far
+ * under the 2^-46 at which a folded fp32 score could round differently.
+ */
+
+static void build_lse_table(double *tab) {
+    const int n = OFK_LSE_COEFS; /* nodes = coefficients */
+    const long double pi = 3.14159265358979323846264338327950288L;
+    for (int cell = 0; cell < OFK_LSE_CELLS; ++cell) {
+        const long double centre = 0.25L * cell + 0.125L;
+        long double x[OFK_LSE_COEFS], dd[OFK_LSE_COEFS], mono[OFK_LSE_COEFS], basis[OFK_LSE_COEFS];
+        for (int j = 0; j < n; ++j) {
+            x[j] = cosl(pi * (2 * j + 1) / (2.0L * n)); /* s in [-1, 1], gap = centre + s / 8 */
+            dd[j] = log1pl(expl(-(centre + x[j] / 8.0L)));
+        }
+        for (int k = 1; k < n; ++k) /* Newton divided differences */
+            for (int j = n - 1; j >= k; --j) dd[j] = (dd[j] - dd[j - 1]) / (x[j] - x[j - k]);
+        for (int j = 0; j < n; ++j) mono[j] = 0, basis[j] = 0;
+        basis[0] = 1; /* basis = prod_{m<k} (s - x[m]) as monomials */
+        for (int k = 0; k < n; ++k) {
+            for (int j = 0; j < n; ++j) mono[j] += dd[k] * basis[j];
+            for (int j = n - 1; j >= 1; --j) basis[j] = basis[j - 1] - x[k] * basis[j];
+            basis[0] = -x[k] * basis[0];
+        }
+        for (int j = 0; j < n; ++j) tab[cell * n + j] = (double)mono[j];
+    }
+}
+
+void openfish_amd_lse_table(double *out) { build_lse_table(out); }
+
 /* ---- gpubuf ---------------------------------------------------------------- */
 
 #define OFA_MAGIC 0x6f66616d64677075ull /* "ofamdgpu" */
@@ -90,6 +124,7 @@ typedef struct {
     int T, N, state_len;
     void *slab;            /* one device allocation behind all pub fields */
     unsigned char *h_out;  /* pinned staging for moves | sequence | qstring */
+    double *lse_table;     /* device copy of the log(1 + e^-gap) table */
     hipStream_t s_main, s_side;
     hipEvent_t ev[EV_COUNT];
     float ms[OPENFISH_AMD_STAGE_COUNT];
@@ -137,6 +172,12 @@ openfish_gpubuf_t *openfish_gpubuf_init(const int T, const int N, const int stat
         p += round_up(sz[i]);
     }
     HIP_OK(hipHostMalloc((void **)&g->h_out, 3 * nt, hipHostMallocDefault));
+    {
+        double tab[OFK_LSE_DOUBLES];
+        build_lse_table(tab);
+        HIP_OK(hipMalloc((void **)&g->lse_table, sizeof tab));
+        HIP_OK(hipMemcpy(g->lse_table, tab, sizeof tab, hipMemcpyHostToDevice));
+    }
     HIP_OK(hipStreamCreateWithFlags(&g->s_main, hipStreamNonBlocking));
     HIP_OK(hipStreamCreateWithFlags(&g->s_side, hipStreamNonBlocking));
     for (int i = 0; i < EV_COUNT; ++i) HIP_OK(hipEventCreate(&g->ev[i]));
@@ -151,6 +192,7 @@ void openfish_gpubuf_free(openfish_gpubuf_t *gpubuf) {
     HIP_OK(hipStreamDestroy(g->s_main));
     HIP_OK(hipStreamDestroy(g->s_side));
     HIP_OK(hipHostFree(g->h_out));
+    HIP_OK(hipFree(g->lse_table));
     HIP_OK(hipFree(g->slab));
     g->magic = 0;
     free(g);
@@ -284,7 +326,7 @@ void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC
     HIP_OK(hipEventRecord(g->ev[EV_BEAM_START], g->s_side));
     launch_ok(ofk_beam_search(scores_TNC, g->pub.bwd_NTC, (ofk_beam_slot_t *)g->pub.beam_vector,
                               (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, log_beam_cut(options),
-                              stay, g->s_side), "beam_search");
+                              stay, g->lse_table, g->s_side), "beam_search");
     HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_side));
 
     launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->s_main),
@@ -338,7 +380,8 @@ void openfish_amd_beam_search(int T, int N, int C, const void *scores, int state
     check_scores(T, N, C, scores, state_len, options);
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     launch_ok(ofk_beam_search(scores, bwd, (ofk_beam_slot_t *)g->pub.beam_vector, (int32_t *)g->pub.states,
-                              g->pub.moves, T, N, state_len, log_beam_cut(options), options->blank_score, NULL),
+                              g->pub.moves, T, N, state_len, log_beam_cut(options), options->blank_score,
+                              g->lse_table, NULL),
               "beam_search");
     HIP_OK(hipStreamSynchronize(0));
 }
@@ -362,7 +405,7 @@ void openfish_amd_decode_from_tensors(int T, int N, int C, const void *scores, i
     join_null_stream(g);
     launch_ok(ofk_beam_search(scores, bwd, (ofk_beam_slot_t *)g->pub.beam_vector, (int32_t *)g->pub.states,
                               g->pub.moves, T, N, state_len, log_beam_cut(options), options->blank_score,
-                              g->s_main), "beam_search");
+                              g->lse_table, g->s_main), "beam_search");
     launch_ok(ofk_sequence(post, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data, g->pub.base_probs,
                            g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N, state_len,
                            phred_for(g, options), g->s_main), "sequence");

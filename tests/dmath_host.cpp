@@ -28,6 +28,30 @@ double max_rel_err_log(const float *s, long n) {
     return worst;
 }
 
+// largest absolute error of log1p_exp_neg against log1pl(expl(-gap))
+double max_abs_err_lse2(const float *gap, long n) {
+    double worst = 0;
+    for (long i = 0; i < n; ++i) {
+        const long double want = log1pl(expl(-(long double)gap[i]));
+        const double err = (double)fabsl((long double)ofa::log1p_exp_neg(gap[i]) - want);
+        if (err > worst) worst = err;
+    }
+    return worst;
+}
+
+// log(e^x + e^y) as the CPU path computes it vs. with log1p_exp_neg: count of differing results
+long lse2_mismatches(const float *xy, long n) {
+    long bad = 0;
+    for (long i = 0; i < n; ++i) {
+        const float x = xy[2 * i], y = xy[2 * i + 1];
+        const float gap = fabsf(x - y), top = x > y ? x : y;
+        const float a = (float)((double)top + (gap < 17.0f ? log(1.0 + exp(-(double)gap)) : 0.0));
+        const float b = (float)((double)top + (gap < 17.0f ? ofa::log1p_exp_neg(gap) : 0.0));
+        if (memcmp(&a, &b, 4) != 0) ++bad;
+    }
+    return bad;
+}
+
 // the CPU path's own arithmetic (libm exp/log in double, fp32 running sum)
 static float lse5_libm(const float v[5], float m) {
     float acc = 0.0f;

@@ -22,6 +22,10 @@ def lib(tmp_path_factory):
     L.max_rel_err_exp.argtypes = [fp, C.c_long]
     L.max_rel_err_log.restype = C.c_double
     L.max_rel_err_log.argtypes = [fp, C.c_long]
+    L.max_abs_err_lse2.restype = C.c_double
+    L.max_abs_err_lse2.argtypes = [fp, C.c_long]
+    L.lse2_mismatches.restype = C.c_long
+    L.lse2_mismatches.argtypes = [fp, C.c_long]
     L.lse5_mismatches.restype = C.c_long
     L.lse5_mismatches.argtypes = [fp, C.c_long]
     return L
@@ -58,3 +62,12 @@ def test_lse5_reproduces_the_libm_roundings(lib, centre, spread):
     rng = np.random.default_rng(int(centre) + 7)
     v = (centre + spread * rng.standard_normal((1000000, 5))).astype(np.float32)
     assert lib.lse5_mismatches(fptr(v), v.shape[0]) == 0
+
+
+def test_pairwise_log_sum_exp_correction(lib):
+    rng = np.random.default_rng(3)
+    gap = np.concatenate([17 * rng.random(500000), 1e-3 * rng.random(50000), [0.0, 16.999998, 1e-30]]).astype(np.float32)
+    assert lib.max_abs_err_lse2(fptr(gap), gap.size) < 2.0 ** -46
+    for centre in (0.0, 40.0, 6000.0):
+        xy = (centre + 5 * rng.standard_normal((1000000, 2))).astype(np.float32)
+        assert lib.lse2_mismatches(fptr(xy), xy.shape[0]) == 0
