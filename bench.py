@@ -86,6 +86,8 @@ def main():
     ap.add_argument("--scan-mode", default="precise", choices=("precise", "fast"))
     ap.add_argument("--cpu-sample", type=int, default=64, help="chunks timed on the CPU path (0 = skip)")
     ap.add_argument("--seed", type=int, default=20251125)
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
+                    help="also run the plain copy kernel once over this many MiB (counter calibration)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this decoder runs on one GPU; chunks are independent, so more GPUs means "
@@ -107,6 +109,14 @@ def main():
     opt = api.DECODER_INIT(q_scale=q_scale, q_shift=q_shift)
     scores = api.upload_scores_to_hip(s16)
     gpubuf = api.GpuBuf(T, N, state_len)
+
+    if a.calibrate_copy:
+        nbytes = a.calibrate_copy << 20
+        src, dst = api.DeviceBuffer(nbytes), api.DeviceBuffer(nbytes)
+        src.fill(1)
+        api.lib().openfish_amd_copy(dst.ptr, src.ptr, nbytes)
+        src.free()
+        dst.free()
 
     for _ in range(a.warmup):
         api.openfish_decode_gpu(T, N, C, scores, state_len, opt, gpubuf)

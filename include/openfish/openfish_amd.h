@@ -38,6 +38,9 @@ void openfish_amd_memcpy_h2d(void *dev, const void *host, size_t bytes);
 void openfish_amd_memcpy_d2h(void *host, const void *dev, size_t bytes);
 void openfish_amd_memset(void *dev, int value, size_t bytes);
 void openfish_amd_sync(void);
+/* device-to-device copy by a plain kernel (reads `bytes`, writes `bytes`; multiple of 16):
+ * the kernel of known traffic against which hardware counters are calibrated */
+void openfish_amd_copy(void *dst, const void *src, size_t bytes);
 /* number of visible devices; 0 when there is none (never exits) */
 int openfish_amd_device_count(void);
 

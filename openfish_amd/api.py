@@ -71,6 +71,7 @@ _SIGS = {
     "openfish_amd_memcpy_d2h": (None, [_vp, _vp, _sz]),
     "openfish_amd_memset": (None, [_vp, _i, _sz]),
     "openfish_amd_sync": (None, []),
+    "openfish_amd_copy": (None, [_vp, _vp, _sz]),
     "openfish_amd_device_count": (_i, []),
     "openfish_amd_bwd_scan": (None, [_i, _i, _i, _vp, _i, _f, _vp]),
     "openfish_amd_fwd_post_scan": (None, [_i, _i, _i, _vp, _i, _f, _vp, _vp]),

@@ -53,6 +53,8 @@ typedef struct {
 int ofk_sequence(const float *post, int32_t *states, const uint8_t *moves, float *qual_data,
                  float *base_probs, float *total_probs, char *sequence, char *qstring, int T, int N,
                  int state_len, const ofk_phred_table_t *phred, void *stream);
+/* device-to-device copy of `bytes` (a multiple of 16); the calibration kernel for counters */
+int ofk_copy(void *dst, const void *src, size_t bytes, void *stream);
 int ofk_rotary_emb(void *x, const float *sin_buf, const float *cos_buf, int batch, int seqlen,
                    int nheads, int rotary_half, long stride_batch, long stride_seq, long stride_head,
                    void *stream);

@@ -486,6 +486,10 @@ void openfish_amd_memcpy_h2d(void *dev, const void *host, size_t bytes) { HIP_OK
 void openfish_amd_memcpy_d2h(void *host, const void *dev, size_t bytes) { HIP_OK(hipMemcpy(host, dev, bytes, hipMemcpyDeviceToHost)); }
 void openfish_amd_memset(void *dev, int value, size_t bytes) { HIP_OK(hipMemset(dev, value, bytes)); }
 void openfish_amd_sync(void) { HIP_OK(hipDeviceSynchronize()); }
+void openfish_amd_copy(void *dst, const void *src, size_t bytes) {
+    launch_ok(ofk_copy(dst, src, bytes, NULL), "copy");
+    HIP_OK(hipStreamSynchronize(0));
+}
 
 int openfish_amd_device_count(void) {
     int n = 0;
