@@ -166,17 +166,6 @@ struct RowRegs {
     }
 };
 
-#ifdef OFK_BEAM_PROFILE
-__device__ unsigned long long g_beam_prof[16];
-#define PROF_MARK(k)                                              \
-    do {                                                          \
-        const unsigned long long now_ = __builtin_amdgcn_s_memtime(); \
-        prof_[k] += now_ - last_;                                 \
-        last_ = now_;                                             \
-    } while (0)
-#else
-#define PROF_MARK(k) do { } while (0)
-#endif
 
 template <int S>
 struct BeamCfg {
@@ -189,9 +178,9 @@ struct BeamCfg {
 // one beam element as handed from one time step to the next
 struct __attribute__((aligned(16))) Elem {
     uint32_t hash;
-    float score;
+    float score;    // candidate score, guide term of its state included
     uint32_t info;  // state | prev << 16 | stay << 21
-    uint32_t pad;
+    float rest;     // score minus that guide term: what the next time step starts from
 };
 // mailbox of one step candidate (index 4i+b): its score, and the stay that claims it
 struct __attribute__((aligned(16))) SlotRec {
@@ -312,7 +301,7 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
         const float thr = key_float(prefix);
         if (lane < kW) {
             sh.hash[lane] = 0;
-            sh.elem[lane] = Elem{0u, 0.f, 0u, 0u};
+            sh.elem[lane] = Elem{0u, 0.f, 0u, 0.f};
         }
         sh.rec[lane].tag = 0;  // tags of real time steps start at 1 << 5
         sh.rec[lane + 64].tag = 0;
@@ -328,7 +317,7 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
                 const uint32_t s = (uint32_t)(j * 64 + lane);
                 const uint32_t hs = crc32_word(kSeed, s);
                 sh.hash[rank] = hs;
-                sh.elem[rank] = Elem{hs, 0.f, s, 0u};
+                sh.elem[rank] = Elem{hs, 0.f, s, 0.f};
             }
             taken += popc64(m);
         }
@@ -347,22 +336,16 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
     ofk_beam_slot_t *bv = beam + (size_t)n * (size_t)(T + 1) * kW;
     if (lane < kW) bv[lane] = (ofk_beam_slot_t)state;
 
-#ifdef OFK_BEAM_PROFILE
-    unsigned long long prof_[16] = {0};
-    unsigned long long last_ = __builtin_amdgcn_s_memtime();
-#endif
     // The search is a chain of dependent short instructions; when it shares a SIMD with
     // throughput-bound waves (the forward scan runs at the same time) it should win the
     // issue arbitration.
     __builtin_amdgcn_s_setprio(3);
     int rows_ready = 0;  // last value seen of the loader's counter; it is usually several rows ahead
     for (int t = 0; t < T; ++t) {
-        PROF_MARK(0);
         while (rows_ready <= t) {
             rows_ready = observe(&sh.ready);
             if (rows_ready <= t) __builtin_amdgcn_s_sleep(1);
         }
-        PROF_MARK(1);
         const int slot = t % LR;
         const _Float16 *rs = row_s[slot];
         const float *rb = row_b[slot];
@@ -386,7 +369,6 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
         my_rec[0].step = c0;
         my_rec[1].step = c1;
 
-        PROF_MARK(2);
         // which previous element j has hash_j == crc^-1(hash_i, last base of i)
         uint32_t match;
         {
@@ -402,12 +384,15 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
                 m |= (x.w == want ? 1u : 0u) << (4 * qd + 3);
             }
             m <<= 16 * h;
-            m |= (uint32_t)__shfl_xor((int)m, 32);
+            {
+                // both halves of the wave looked at 16 hashes each: lanes i and i+32 join their masks
+                const auto both = __builtin_amdgcn_permlane32_swap(m, m, false, false);
+                m = both[0] | both[1];
+            }
             const uint32_t live = w >= 32 ? 0xFFFFFFFFu : ((1u << w) - 1u);
             match = valid ? (m & live) : 0u;
         }
 
-        PROF_MARK(3);
         // merge stays with the step spelling the same sequence (src/beam_search.c:281-316).
         // The stay posts its score into the mailbox of the step it matches; then both
         // sides read each other's score and apply their half of the merge.
@@ -469,19 +454,21 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
                     if (st1 > c1) c1 = -FLT_MAX; else pend |= 4u;
                 }
                 while (ballot(pend != 0) != 0) {
-                    const unsigned pick = pend & (0u - pend);
-                    const float x = pick == 1u ? cs : pick == 2u ? st0 : st1;
-                    const float y = pick == 1u ? other : pick == 2u ? c0 : c1;
-                    const float folded = log_sum_exp(x, y, sh.lse);
-                    if (pick == 1u) cs = folded;
-                    if (pick == 2u) c0 = folded;
-                    if (pick == 4u) c1 = folded;
-                    pend ^= pick;
+                    // only the lanes that have a fold to do touch the coefficient table
+                    if (pend != 0) {
+                        const unsigned pick = pend & (0u - pend);
+                        const float x = pick == 1u ? cs : pick == 2u ? st0 : st1;
+                        const float y = pick == 1u ? other : pick == 2u ? c0 : c1;
+                        const float folded = log_sum_exp(x, y, sh.lse);
+                        if (pick == 1u) cs = folded;
+                        if (pick == 2u) c0 = folded;
+                        if (pick == 4u) c1 = folded;
+                        pend ^= pick;
+                    }
                 }
             }
         }
 
-        PROF_MARK(4);
         // cut-off (src/beam_search.c:320-381)
         float best = -FLT_MAX;
         if (valid) best = fmaxf(c0, c1);
@@ -518,7 +505,6 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
             if (kept > kW) kept = kW;
         }
 
-        PROF_MARK(5);
         // survivors in candidate order: steps (i, b) by i then b, then stays by i
         {
             const int before = popc64(k0 & below) + popc64(k1 & below);
@@ -531,31 +517,32 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
             const uint32_t from = (uint32_t)i << 16;
             if (keep0 && rank0 < kW) {
                 sh.hash[rank0] = h0;
-                sh.elem[rank0] = Elem{h0, c0, (uint32_t)(lo4 + b0) | from, 0u};
+                sh.elem[rank0] = Elem{h0, c0, (uint32_t)(lo4 + b0) | from, c0 - g01.x};
             }
             if (keep1 && rank1 < kW) {
                 sh.hash[rank1] = h1;
-                sh.elem[rank1] = Elem{h1, c1, (uint32_t)(lo4 + b0 + 1) | from, 0u};
+                sh.elem[rank1] = Elem{h1, c1, (uint32_t)(lo4 + b0 + 1) | from, c1 - g01.y};
             }
             if (keeps && ranks < kW) {
                 sh.hash[ranks] = hash;
-                sh.elem[ranks] = Elem{hash, cs, (uint32_t)state | from | (1u << 21), 0u};
+                sh.elem[ranks] = Elem{hash, cs, (uint32_t)state | from | (1u << 21), cs - gst};
             }
             wave_fence();
         }
         w = kept;
+        float rest = 0.f;
         if (i < w) {
             const Elem e = sh.elem[i];
             hash = e.hash;
             score = e.score;
             info = e.info;
+            rest = e.rest;
         } else {
             score = 0.f;
             info = 0;
         }
         state = (int)(info & 0xFFFFu);
 
-        PROF_MARK(6);
         // last block: the best survivor goes to slot 0 (src/beam_search.c:398-414)
         if (t == T - 1) {
             const bool in = i < w;
@@ -565,25 +552,24 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
             if (arg != 0) {
                 const uint32_t hash0 = lane_u(hash, 0), hasha = lane_u(hash, arg);
                 const uint32_t in0 = lane_u(info, 0), ina = lane_u(info, arg);
-                const float sc0 = lane_f(score, 0), sca = lane_f(score, arg);
-                if (i == 0) { hash = hasha; info = ina; score = sca; }
-                if (i == arg) { hash = hash0; info = in0; score = sc0; }
+                const float re0 = lane_f(rest, 0), rea = lane_f(rest, arg);
+                if (i == 0) { hash = hasha; info = ina; rest = rea; }
+                if (i == arg) { hash = hash0; info = in0; rest = re0; }
                 state = (int)(info & 0xFFFFu);
             }
         }
 
-        // drop the guide term again and persist the slot (src/beam_search.c:417-427)
+        // drop the guide term again and persist the slot (src/beam_search.c:417-427); the
+        // difference was taken by the lane that held the candidate, which had the term at hand
+        score = rest;
         if (i < w) {
-            score = score - rb[state];
             if (h == 0)
                 bv[(size_t)(t + 1) * kW + i] =
                     (ofk_beam_slot_t)((uint32_t)state | (((info >> 16) & 31u) << 10) | (((info >> 21) & 1u) << 15));
         }
-        PROF_MARK(7);
         publish(&sh.consumed, t + 1);
     }
 
-    PROF_MARK(7);
     // ---- traceback from slot 0 of the last block (src/beam_search.c:432-439) ----
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -612,11 +598,6 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
         }
         wave_fence();
     }
-#ifdef OFK_BEAM_PROFILE
-    PROF_MARK(8);
-    if (blockIdx.x == 0 && lane == 0)
-        for (int k = 0; k < 16; ++k) g_beam_prof[k] = prof_[k];
-#endif
 }
 
 template <int S>
@@ -634,11 +615,6 @@ int g_beam_flags = 0;
 
 extern "C" void ofk_set_beam_flags(int flags) { g_beam_flags = flags; }
 
-#ifdef OFK_BEAM_PROFILE
-extern "C" void ofk_beam_profile(unsigned long long *out16) {
-    (void)hipMemcpyFromSymbol(out16, HIP_SYMBOL(g_beam_prof), sizeof(unsigned long long) * 16);
-}
-#endif
 
 extern "C" int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                                uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
