@@ -1,9 +1,12 @@
 // Double-precision exp and log for the scans, written for the narrow domains the
 // scans need so that they cost a few dozen full-rate fp64 FMAs instead of a
 // general libm call:
-//   exp_nonpos(d) : e^d for a float d <= 0, relative error below 2^-46
-//   log_1to5(s)   : ln(s) for a float s in [1, 5] (a sum of five terms <= 1, one of
-//                   which is exactly 1), relative error below 2^-51
+//   exp_nonpos(d)   : e^d for a float d <= 0, relative error below 2^-46
+//   log_1to5(s)     : ln(s) for a float s in [1, 5] (a sum of five terms <= 1, one of
+//                     which is exactly 1), relative error below 2^-51
+//   log_1to5_tab(s) : the same from a 32-entry table of (1/c, ln c), absolute error
+//                     below 2^-51; half the instructions
+//   log1p_exp_neg   : ln(1 + e^-gap), the pairwise log-sum-exp correction
 // The CPU path evaluates exp and log in double and then rounds to fp32 (reference
 // src/decode_cpu.c:45-49); these stand in for its libm calls.  With the errors above
 // a result can round to a different fp32 value only when the exact value lies
@@ -77,6 +80,33 @@ OFA_HD double exp_nonpos(float d) {
     return double_of(scaled);
 }
 
+// The same without the clamp: the scaling is a true ldexp, which underflows to zero by
+// itself.  Needs |d| < 1e9 (the integer part of d*log2(e) is read from 32 bits).
+OFA_HD double exp_nonpos_ldexp(float d) {
+    const double x = (double)d;
+    const double kShift = 6755399441055744.0;
+    const double kLog2e = 1.4426950408889634074;
+    const double kLn2Hi = 6.93147180369123816490e-01;
+    const double kLn2Lo = 1.90821492927058770002e-10;
+    const double t = __builtin_fma(x, kLog2e, kShift);
+    const double n = t - kShift;
+    double r = __builtin_fma(n, -kLn2Hi, x);
+    r = __builtin_fma(n, -kLn2Lo, r);
+    double p = 1.0 / 39916800.0;
+    p = __builtin_fma(p, r, 1.0 / 3628800.0);
+    p = __builtin_fma(p, r, 1.0 / 362880.0);
+    p = __builtin_fma(p, r, 1.0 / 40320.0);
+    p = __builtin_fma(p, r, 1.0 / 5040.0);
+    p = __builtin_fma(p, r, 1.0 / 720.0);
+    p = __builtin_fma(p, r, 1.0 / 120.0);
+    p = __builtin_fma(p, r, 1.0 / 24.0);
+    p = __builtin_fma(p, r, 1.0 / 6.0);
+    p = __builtin_fma(p, r, 0.5);
+    p = __builtin_fma(p, r, 1.0);
+    p = __builtin_fma(p, r, 1.0);
+    return __builtin_ldexp(p, (int)(uint32_t)bits_of(t));
+}
+
 // k*ln2 + ln(1 + f) for f in [sqrt(1/2) - 1, sqrt(2) - 1]:
 // ln(1 + f) = 2 atanh(z), z = f / (2 + f), |z| <= 0.1716.
 OFA_HD double log_core(double f, int k) {
@@ -116,6 +146,39 @@ OFA_HD double log_1to5(float s) {
     return log_core((double)u - 1.0, k);  // the difference is exact
 }
 
+// Table-driven ln(s), s a float in [1, 5].  The mantissa interval [1, 2) is cut into 32
+// cells with centres c_i = 1 + (2i + 1)/64; entry i holds inv = fl(1/c_i) and
+// lnc = -ln(inv).  For s = 2^k * u:  ln(s) = k ln2 + lnc + log1p(u * inv - 1), and
+// |u * inv - 1| <= 1/64 lets the series stop at the eighth power (next term < 2^-57).
+struct LogCell {
+    double inv, lnc;
+};
+OFA_HD LogCell log_cell(int i) {
+    LogCell c;
+    c.inv = 1.0 / (1.0 + (2 * i + 1) / 64.0);                 // in (0.5, 1)
+    const bool low = c.inv < 0.70710678118654752;
+    c.lnc = -log_core(low ? 2.0 * c.inv - 1.0 : c.inv - 1.0, low ? -1 : 0);  // differences exact
+    return c;
+}
+OFA_HD double log_1to5_tab(float s, const LogCell *table) {
+    const uint32_t b = bits_of(s);
+    const int k = (int)(b >> 23) - 127;
+    const LogCell c = table[(b >> 18) & 31u];
+    const double u = (double)float_of((b & 0x007fffffu) | 0x3f800000u);
+    const double r = __builtin_fma(u, c.inv, -1.0);
+    double q = -1.0 / 8.0;
+    q = __builtin_fma(q, r, 1.0 / 7.0);
+    q = __builtin_fma(q, r, -1.0 / 6.0);
+    q = __builtin_fma(q, r, 1.0 / 5.0);
+    q = __builtin_fma(q, r, -1.0 / 4.0);
+    q = __builtin_fma(q, r, 1.0 / 3.0);
+    q = __builtin_fma(q, r, -0.5);
+    q = __builtin_fma(q, r, 1.0);
+    const double lu = __builtin_fma(q, r, c.lnc);
+    const double kLn2 = 0.69314718055994530942;
+    return __builtin_fma((double)k, kLn2, lu);
+}
+
 // ln(1 + e^-gap) for a float gap in [0, 17): the correction term of log(e^x + e^y)
 // (reference src/beam_search.c:43-47), absolute error below 2^-46
 OFA_HD double log1p_exp_neg(float gap) {
@@ -134,6 +197,17 @@ OFA_HD float lse5_cpu_rounding(float v0, float v1, float v2, float v3, float v4,
     s = (float)((double)s + exp_nonpos(v3 - m));
     s = (float)((double)s + exp_nonpos(v4 - m));
     return (float)((double)m + log_1to5(s));
+}
+
+// the same update with the table-driven logarithm and the ldexp-scaled exponential
+OFA_HD float lse5_cpu_rounding_tab(float v0, float v1, float v2, float v3, float v4, float m,
+                                   const LogCell *table) {
+    float s = (float)exp_nonpos_ldexp(v0 - m);
+    s = (float)((double)s + exp_nonpos_ldexp(v1 - m));
+    s = (float)((double)s + exp_nonpos_ldexp(v2 - m));
+    s = (float)((double)s + exp_nonpos_ldexp(v3 - m));
+    s = (float)((double)s + exp_nonpos_ldexp(v4 - m));
+    return (float)((double)m + log_1to5_tab(s, table));
 }
 
 }  // namespace ofa

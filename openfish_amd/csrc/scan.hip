@@ -82,10 +82,10 @@ __device__ __forceinline__ float group_max(float x) {
 
 // max + log(sum_i exp(v_i - max)), sum taken in the order v0..v4
 template <bool PRECISE>
-__device__ __forceinline__ float lse5(float v0, float v1, float v2, float v3, float v4) {
+__device__ __forceinline__ float lse5(float v0, float v1, float v2, float v3, float v4, const ofa::LogCell *logtab) {
     const float m = fmaxf(fmaxf(fmaxf(v0, v1), v2), fmaxf(v3, v4));
     if constexpr (PRECISE) {
-        return ofa::lse5_cpu_rounding(v0, v1, v2, v3, v4, m);
+        return ofa::lse5_cpu_rounding_tab(v0, v1, v2, v3, v4, m, logtab);
     } else {
         float s = __builtin_amdgcn_exp2f((v0 - m) * kLog2e);
         s += __builtin_amdgcn_exp2f((v1 - m) * kLog2e);
@@ -214,21 +214,22 @@ struct FloatRun {
 };
 
 template <int I, int SPL, bool PRECISE>
-__device__ __forceinline__ void bwd_update(float (&a)[SPL], const float4 &nx, const BwdRow<SPL> &row, float stay) {
+__device__ __forceinline__ void bwd_update(float (&a)[SPL], const float4 &nx, const BwdRow<SPL> &row, float stay,
+                                           const ofa::LogCell *logtab) {
     if constexpr (I < SPL) {
         a[I] = lse5<PRECISE>(a[I] + stay, nx.x + row.template get<0, I>(), nx.y + row.template get<1, I>(),
-                             nx.z + row.template get<2, I>(), nx.w + row.template get<3, I>());
-        bwd_update<I + 1, SPL, PRECISE>(a, nx, row, stay);
+                             nx.z + row.template get<2, I>(), nx.w + row.template get<3, I>(), logtab);
+        bwd_update<I + 1, SPL, PRECISE>(a, nx, row, stay, logtab);
     }
 }
 
 template <int I, int SPL, bool PRECISE>
 __device__ __forceinline__ void fwd_update(float (&f)[SPL], float p0, float p1, float p2, float p3,
-                                           const FwdRow<SPL> &row, float stay) {
+                                           const FwdRow<SPL> &row, float stay, const ofa::LogCell *logtab) {
     if constexpr (I < SPL) {
         f[I] = lse5<PRECISE>(f[I] + stay, p0 + row.template get<I, 0>(), p1 + row.template get<I, 1>(),
-                             p2 + row.template get<I, 2>(), p3 + row.template get<I, 3>());
-        fwd_update<I + 1, SPL, PRECISE>(f, p0, p1, p2, p3, row, stay);
+                             p2 + row.template get<I, 2>(), p3 + row.template get<I, 3>(), logtab);
+        fwd_update<I + 1, SPL, PRECISE>(f, p0, p1, p2, p3, row, stay, logtab);
     }
 }
 
@@ -243,8 +244,10 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
     constexpr int Q = Sh::kQuarter;
     constexpr int H = 4 / SPL;  // lanes sharing one quad
     __shared__ __attribute__((aligned(16))) float vec[Sh::kChunks][2][S];
+    __shared__ __attribute__((aligned(16))) ofa::LogCell logtab[32];
 
     const int tid = threadIdx.x;
+    if (PRECISE && tid < 32) logtab[tid] = ofa::log_cell(tid);
     const int g = tid / L, l = tid % L;
     const int r = l / H, c0 = (l % H) * SPL;  // own states: r + (c0 + i) * Q
     int n = blockIdx.x * Sh::kChunks + g;
@@ -273,6 +276,7 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
     int buf = 0;
 #pragma unroll
     for (int i = 0; i < SPL; ++i) vec[g][0][r + (c0 + i) * Q] = 0.f;
+    __syncthreads();  // the log table is shared by the whole group
 
     for (int done = 0; done < T; done += DEPTH) {
 #pragma unroll
@@ -283,7 +287,7 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
                 if (t - DEPTH >= 0) ring[k].load(sp + (size_t)(t - DEPTH) * row_stride);
                 chunk_sync<Sh::kMultiWave>();
                 const float4 nx = *reinterpret_cast<const float4 *>(&vec[g][buf][4 * r]);
-                bwd_update<0, SPL, PRECISE>(a, nx, row, stay);
+                bwd_update<0, SPL, PRECISE>(a, nx, row, stay, logtab);
                 buf ^= 1;
 #pragma unroll
                 for (int i = 0; i < SPL; ++i) vec[g][buf][r + (c0 + i) * Q] = a[i];
@@ -308,8 +312,10 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
     constexpr int Q = Sh::kQuarter;
     __shared__ __attribute__((aligned(16))) float vec[Sh::kChunks][2][S];
     __shared__ float part[2][Sh::kChunks][Sh::kChunkWaves];
+    __shared__ __attribute__((aligned(16))) ofa::LogCell logtab[32];
 
     const int tid = threadIdx.x;
+    if (PRECISE && tid < 32) logtab[tid] = ofa::log_cell(tid);
     const int g = tid / L, l = tid % L;
     const int s0 = SPL * l, q = s0 >> 2;  // own states s0 .. s0+SPL-1, all in quad q
     const int wave = l / 64;  // wave within the chunk
@@ -357,6 +363,7 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
 #pragma unroll
     for (int i = 0; i < SPL; ++i) f[i] = 0.f;
     int buf = 0;
+    __syncthreads();  // the log table is shared by the whole group
 
     for (int done = 0; done <= T; done += DEPTH) {
 #pragma unroll
@@ -401,7 +408,7 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
                     const float p1 = vec[g][buf][q + Q];
                     const float p2 = vec[g][buf][q + 2 * Q];
                     const float p3 = vec[g][buf][q + 3 * Q];
-                    fwd_update<0, SPL, PRECISE>(f, p0, p1, p2, p3, row, stay);
+                    fwd_update<0, SPL, PRECISE>(f, p0, p1, p2, p3, row, stay, logtab);
                     buf ^= 1;
                 }
             }

@@ -26,6 +26,10 @@ def lib(tmp_path_factory):
     L.max_abs_err_lse2.argtypes = [fp, C.c_long]
     L.lse2_mismatches.restype = C.c_long
     L.lse2_mismatches.argtypes = [fp, C.c_long]
+    L.max_rel_err_exp_ldexp.restype = C.c_double
+    L.max_rel_err_exp_ldexp.argtypes = [fp, C.c_long]
+    L.max_abs_err_log_tab.restype = C.c_double
+    L.max_abs_err_log_tab.argtypes = [fp, C.c_long]
     L.lse5_mismatches.restype = C.c_long
     L.lse5_mismatches.argtypes = [fp, C.c_long]
     return L
@@ -40,6 +44,17 @@ def test_exp_relative_error_below_2_pow_minus_46(lib):
     d = np.concatenate([-80 * rng.random(400000), -rng.random(200000), -1e-3 * rng.random(100000),
                         -(np.arange(0, 2560) / 32.0), [0.0, -0.0, -1e-30, -79.99999]]).astype(np.float32)
     assert lib.max_rel_err_exp(fptr(d), d.size) < 2.0 ** -46
+
+
+def test_ldexp_scaled_exp_and_table_log(lib):
+    rng = np.random.default_rng(4)
+    d = np.concatenate([-100 * rng.random(400000), -rng.random(100000), [0.0, -700.0]]).astype(np.float32)
+    assert lib.max_rel_err_exp_ldexp(fptr(d), d.size) < 2.0 ** -46
+    far = np.array([-745.0, -20000.0, -1e8], np.float32)  # subnormal or zero results: absolute check
+    assert lib.max_rel_err_exp_ldexp(fptr(far[1:]), 2) == 0.0  # exactly zero, like exp()
+    s = np.concatenate([1 + 4 * rng.random(500000), 1 + 1e-4 * rng.random(100000),
+                        [1.0, 5.0, 2.0, 4.0, 1.015625, 1.9999999, 3.9999998]]).astype(np.float32)
+    assert lib.max_abs_err_log_tab(fptr(s), s.size) < 2.0 ** -51
 
 
 def test_exp_of_zero_is_exactly_one_and_far_tail_is_tiny(lib):
