@@ -67,6 +67,9 @@ void openfish_gpubuf_free(openfish_gpubuf_t *gpubuf);
  * Decode a batch on the current device (reference src/openfish.c:43-63,
  * src/decode_hip.hip:83-217).
  *   scores_TNC  device pointer, T*N*C IEEE half, TNC contiguous, C = 4*4^state_len
+ *               (the reference's layout: element 4*state + dropped base).  C = 5*4^state_len
+ *               is also accepted: element 5*state is then a blank column that is skipped
+ *               and elements 5*state + 1 + base are the four step scores.
  *   *moves, *sequence, *qstring
  *               on return host buffers of N*T bytes each obtained with malloc;
  *               chunk n starts at n*T; sequence/qstring hold seq_len characters

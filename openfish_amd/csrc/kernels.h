@@ -55,6 +55,9 @@ int ofk_sequence(const float *post, int32_t *states, const uint8_t *moves, float
                  int state_len, const ofk_phred_table_t *phred, void *stream);
 /* device-to-device copy of `bytes` (a multiple of 16); the calibration kernel for counters */
 int ofk_copy(void *dst, const void *src, size_t bytes, void *stream);
+/* fp16 [groups][5] -> [groups][4], dropping element 0 of every group (the blank column of a
+ * five-column CRF head); groups = T * N * S */
+int ofk_drop_blank_column(const void *scores5, void *scores4, size_t groups, void *stream);
 int ofk_rotary_emb(void *x, const float *sin_buf, const float *cos_buf, int batch, int seqlen,
                    int nheads, int rotary_half, long stride_batch, long stride_seq, long stride_head,
                    void *stream);

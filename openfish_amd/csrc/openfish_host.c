@@ -125,6 +125,8 @@ typedef struct {
     void *slab;            /* one device allocation behind all pub fields */
     unsigned char *h_out;  /* pinned staging for moves | sequence | qstring */
     double *lse_table;     /* device copy of the log(1 + e^-gap) table */
+    void *scores4;         /* four-column copy of a five-column score tensor, allocated on first use */
+    size_t scores4_bytes;
     hipStream_t s_main, s_side;
     hipEvent_t ev[EV_COUNT];
     float ms[OPENFISH_AMD_STAGE_COUNT];
@@ -193,6 +195,7 @@ void openfish_gpubuf_free(openfish_gpubuf_t *gpubuf) {
     HIP_OK(hipStreamDestroy(g->s_side));
     HIP_OK(hipHostFree(g->h_out));
     HIP_OK(hipFree(g->lse_table));
+    if (g->scores4) HIP_OK(hipFree(g->scores4));
     HIP_OK(hipFree(g->slab));
     g->magic = 0;
     free(g);
@@ -207,12 +210,35 @@ static ofa_gpubuf_t *checked(const openfish_gpubuf_t *gpubuf, int T, int N, int 
     return g;
 }
 
-static void check_scores(int T, int N, int C, const void *scores, int state_len, const openfish_opt_t *opt) {
+static void check_scores_any(int T, int N, int C, const void *scores, int state_len, const openfish_opt_t *opt,
+                             int allow_blank_column) {
     check_state_len(state_len);
     if (T < 1 || N < 1) die("T and N must be positive");
-    if (C != 4 * states_of(state_len)) die("C must be 4 * 4^state_len (one score per state and dropped base)");
+    if (C != 4 * states_of(state_len) && !(allow_blank_column && C == 5 * states_of(state_len)))
+        die("C must be 4 * 4^state_len (one score per state and dropped base)");
     if (!scores) die("scores_TNC is NULL");
     if (!opt) die("options is NULL");
+}
+
+static void check_scores(int T, int N, int C, const void *scores, int state_len, const openfish_opt_t *opt) {
+    check_scores_any(T, N, C, scores, state_len, opt, 0);
+}
+
+/* A five-column tensor (C = 5 * 4^state_len: a blank/stay column, then the four step columns
+ * of every state, as a CRF head emits them before the blank is dropped) is reduced to the
+ * four-column layout the decoder consumes; the stay score is options->blank_score, as for
+ * any other input (reference src/beam_search.c:213). */
+static const void *four_columns(ofa_gpubuf_t *g, int T, int N, int C, const void *scores, int state_len) {
+    const size_t S = (size_t)states_of(state_len);
+    if ((size_t)C == 4 * S) return scores;
+    const size_t groups = (size_t)T * (size_t)N * S, bytes = groups * 8;
+    if (g->scores4_bytes < bytes) {
+        if (g->scores4) HIP_OK(hipFree(g->scores4));
+        HIP_OK(hipMalloc(&g->scores4, bytes));
+        g->scores4_bytes = bytes;
+    }
+    launch_ok(ofk_drop_blank_column(scores, g->scores4, groups, g->s_main), "drop_blank_column");
+    return g->scores4;
 }
 
 static float log_beam_cut(const openfish_opt_t *opt) {
@@ -312,13 +338,14 @@ static void join_null_stream(ofa_gpubuf_t *g) {
 void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC, const int state_len,
                          const openfish_opt_t *options, const openfish_gpubuf_t *gpubuf, uint8_t **moves,
                          char **sequence, char **qstring) {
-    check_scores(T, N, C, scores_TNC, state_len, options);
+    check_scores_any(T, N, C, scores_TNC, state_len, options, 1);
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     const float stay = options->blank_score; /* as the reference GPU path, src/decode_hip.hip:120 */
     OPENFISH_LOG_TRACE("scores tensor dim: %d, %d, %d", T, N, C);
 
     join_null_stream(g);
     HIP_OK(hipEventRecord(g->ev[EV_START], g->s_main));
+    scores_TNC = (void *)four_columns(g, T, N, C, scores_TNC, state_len);
     launch_ok(ofk_bwd_scan(scores_TNC, g->pub.bwd_NTC, T, N, state_len, stay, g->s_main), "bwd_scan");
     HIP_OK(hipEventRecord(g->ev[EV_BWD_END], g->s_main));
 

@@ -102,10 +102,10 @@ def run_snippet(code):
 
 
 def test_wrong_channel_count_exits_with_message():
-    # C = 5*S (a blank column) is not what the decoder consumes: message + exit, no GPU touched
+    # a channel count that is neither 4*S nor 5*S: message + exit, no GPU touched
     r = run_snippet("import ctypes as C\nfrom openfish_amd import api\n"
                     "o = api.DECODER_INIT()\nmv, sq, qs = C.c_void_p(), C.c_void_p(), C.c_void_p()\n"
-                    "api.lib().openfish_decode_gpu(10, 2, 320, 4096, 3, C.byref(o), None, C.byref(mv), C.byref(sq), C.byref(qs))\n"
+                    "api.lib().openfish_decode_gpu(10, 2, 300, 4096, 3, C.byref(o), None, C.byref(mv), C.byref(sq), C.byref(qs))\n"
                     "print('survived')")
     assert r.returncode != 0 and "survived" not in r.stdout
     assert "C must be 4 * 4^state_len" in r.stderr

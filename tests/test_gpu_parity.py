@@ -197,6 +197,21 @@ def test_gpubuf_is_reusable_for_smaller_batches(api):
         assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
 
 
+@pytest.mark.parametrize("state_len,T,N", [(3, 150, 5), (4, 90, 3), (5, 40, 2)])
+def test_five_column_input_equals_its_four_column_view(api, state_len, T, N):
+    """C = 5*S: a blank column in front of the four step columns of every state"""
+    S = 4 ** state_len
+    four, five = synth.crf_scores(T, N, state_len, seed=55, five_columns=True)
+    assert np.array_equal(five.reshape(T, N, S, 5)[..., 1:].reshape(T, N, 4 * S), four)
+    kw = dict(q_scale=0.95, q_shift=-0.2)
+    ref = O.decode(four.astype(np.float32), state_len, kw, nthreads=4)
+    gb = api.GpuBuf(T, N, state_len)
+    sc5 = api.upload_scores_to_hip(five)
+    mv, sq, qs = api.openfish_decode_gpu(T, N, 5 * S, sc5, state_len, api.DECODER_INIT(**kw), gb)
+    assert np.array_equal(gb.tensor("bwd_NTC"), ref["bwd"])
+    assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
+
+
 def test_constant_scores_closed_form(api):
     T, N, sl, c = 64, 3, 3, 0.75
     S = 4 ** sl
