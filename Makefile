@@ -6,6 +6,7 @@
 #   make            both libraries
 #   make rocm=1     accepted for compatibility with the reference's invocation
 #   make oracle     the CPU oracle used by the tests (never linked into the libraries)
+#   ./openfish <scores.blob> <N> <state_len>   decode a blob, write moves/sequence/qstring.blob
 
 ROCM_ROOT ?= /opt/rocm
 HIPCC     ?= $(ROCM_ROOT)/bin/hipcc
@@ -25,7 +26,7 @@ LDLIBS   := -L$(ROCM_ROOT)/lib -Wl,-rpath,$(ROCM_ROOT)/lib -lamdhip64 -lm -lpthr
 HIP_OBJ := $(BUILD)/scan.o $(BUILD)/beam.o $(BUILD)/sequence.o $(BUILD)/rotary.o $(BUILD)/copy.o
 C_OBJ   := $(BUILD)/openfish_host.o
 
-all: lib/libopenfish.a openfish_amd/libopenfish_amd.so
+all: lib/libopenfish.a openfish_amd/libopenfish_amd.so openfish
 
 $(BUILD)/%.o: $(SRC)/%.hip $(SRC)/kernels.h $(SRC)/dmath.h
 	@mkdir -p $(BUILD)
@@ -43,10 +44,14 @@ lib/libopenfish.a: $(HIP_OBJ) $(C_OBJ)
 openfish_amd/libopenfish_amd.so: $(HIP_OBJ) $(C_OBJ)
 	$(HIPCC) $(ROCM_ARCH) -shared -fPIC $^ -o $@ $(LDLIBS)
 
+# the command-line driver (the reference's `openfish` test binary), linked against the static library
+openfish: $(SRC)/openfish_cli.c lib/libopenfish.a
+	$(CC) $(CFLAGS) $< lib/libopenfish.a $(LDLIBS) -lstdc++ -o $@
+
 oracle:
 	$(MAKE) -C oracle
 
 clean:
-	rm -rf $(BUILD) lib/libopenfish.a openfish_amd/libopenfish_amd.so
+	rm -rf $(BUILD) lib/libopenfish.a openfish_amd/libopenfish_amd.so openfish
 
 .PHONY: all oracle clean
