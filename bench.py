@@ -36,6 +36,13 @@ WORKLOADS = {
 }
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch in GB, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the plain
+# copy kernel's reading of the same counters (profiles/decode_*.md); keyed by workload and kernel
+MEASURED_TRAFFIC_GB = {
+    ("hac", 512, "bwd"): 2.621, ("hac", 512, "fwd_post"): 3.495, ("hac", 512, "beam"): 2.735,
+    ("hac", 512, "sequence"): 0.694,
+}
+
 
 def algorithmic_bytes(state_len, T, N):
     """bytes each kernel has to move at least once, per launch"""
@@ -76,16 +83,48 @@ def cpu_baseline(s16, state_len, opt_kw, sample_chunks):
                       "median of 3 calls of openfish_decode_cpu (%.3f s each)" % (sample_chunks, T, sec)}
 
 
+def rotary_bench(a):
+    """in-place rotary embedding on the shape the reference's driver sketches
+    (src/main.c:84-95): batch 500, seqlen 833, 8 heads of 64, rotary_half 32, half data"""
+    from openfish_amd import api, synth
+    batch, seqlen, nheads, head_dim, half = 500, 833, 8, 64, 32
+    strides = (seqlen * nheads * head_dim, nheads * head_dim, head_dim)
+    rng = np.random.default_rng(a.seed)
+    x = rng.standard_normal((batch, seqlen, nheads, head_dim), dtype=np.float32).astype(np.float16)
+    sn, cs = synth.rotary_tables(seqlen, half)
+    xd, sd, cd = api.DeviceBuffer.from_host(x), api.DeviceBuffer.from_host(sn), api.DeviceBuffer.from_host(cs)
+    call = lambda: api.openfish_rotary_emb_gpu(xd, sd, cd, batch, seqlen, nheads, head_dim, half, *strides)  # noqa: E731
+    for _ in range(a.warmup):
+        call()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        call()
+    ms = 1e3 * (time.perf_counter() - t0) / a.steps
+    nbytes = 2 * x.nbytes + sn.nbytes + cs.nbytes  # x read and written once, tables read once
+    gbs = nbytes / 1e9 / (ms / 1e3)
+    print(json.dumps({
+        "metric": "rotary embedding, in place, half", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "rotary: batch 500, seqlen 833, 8 heads x 64, rotary_half 32 (half x, fp32 sin/cos); "
+                               "time of the synchronous call, launch and sync included"},
+        "roofline": {"bound": "hbm", "kernel": "rotary_vec8", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+        "cpu_baseline": None}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="hac", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="hac", choices=sorted(WORKLOADS) + ["rotary"])
     ap.add_argument("--chunks", type=int, default=0, help="override N")
     ap.add_argument("--scan-mode", default="precise", choices=("precise", "fast"))
     ap.add_argument("--cpu-sample", type=int, default=64, help="chunks timed on the CPU path (0 = skip)")
     ap.add_argument("--seed", type=int, default=20251125)
+    ap.add_argument("--alt-steps", type=int, default=3,
+                    help="extra timed calls with the hardware-exp scan arithmetic, reported beside the main result (0 = skip)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="also run the plain copy kernel once over this many MiB (counter calibration)")
     a = ap.parse_args()
@@ -96,6 +135,9 @@ def main():
     from openfish_amd import api, synth
     if api.device_count() < 1:
         sys.exit("bench.py: no HIP device visible")
+
+    if a.workload == "rotary":
+        return rotary_bench(a)
 
     state_len, T, N, stress, q_scale, q_shift = WORKLOADS[a.workload]
     if a.chunks:
@@ -143,8 +185,29 @@ def main():
     stages["scan_plus_posterior"] = {"ms": round(scan_ms, 4), "GBps": round(scan_gbs, 1),
                                      "frac_of_hbm_peak": round(scan_gbs / HBM_PEAK_GBS, 4)}
     dominant = max(("bwd", "fwd_post", "beam", "sequence"), key=lambda k: stages[k]["ms"])
+    traffic = MEASURED_TRAFFIC_GB.get((a.workload, N, dominant))
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(stages[dominant]["GBps"] / HBM_PEAK_GBS, 4), "traffic": None}
+                "unit": "GB/s", "frac": round(stages[dominant]["GBps"] / HBM_PEAK_GBS, 4),
+                "traffic": None if traffic is None else round(traffic * 1e9)}
+
+    # the same batch with the hardware-exp/log scan arithmetic, for comparison (not `value`)
+    other = None
+    if a.scan_mode == "precise" and a.alt_steps > 0:
+        api.set_scan_mode(True)
+        alt = {k: [] for k in api.STAGES}
+        api.openfish_decode_gpu(T, N, C, scores, state_len, opt, gpubuf)
+        t1 = time.perf_counter()
+        for _ in range(a.alt_steps):
+            api.openfish_decode_gpu(T, N, C, scores, state_len, opt, gpubuf)
+            for k, v in gpubuf.timings().items():
+                alt[k].append(v)
+        alt_ms = 1e3 * (time.perf_counter() - t1) / a.alt_steps
+        api.set_scan_mode(False)
+        fb, ff = statistics.mean(alt["bwd"]), statistics.mean(alt["fwd_post"])
+        other = {"chunks_per_s": round(N / (alt_ms / 1e3), 1), "ms_per_step": round(alt_ms, 4),
+                 "bwd_ms": round(fb, 4), "fwd_post_ms": round(ff, 4),
+                 "scan_plus_posterior_GBps": round((need["bwd"] + need["fwd_post"]) / 1e9 / ((fb + ff) / 1e3), 1),
+                 "note": "scans with v_exp_f32/v_log_f32: bwd within 2 ulp, a few posteriors per ten million beyond 1e-3 relative"}
 
     opt_kw = dict(beam_cut=100.0, blank_score=2.0, q_shift=q_shift, q_scale=q_scale)
     cpu = cpu_baseline(s16, state_len, opt_kw, min(a.cpu_sample, N)) if a.cpu_sample > 0 else None
@@ -157,7 +220,7 @@ def main():
         "config": {"workload": "%s: state_len %d, S=%d, C=%d fp16 TNC, T=%d, N=%d, beam 32, beam_cut 100, blank 2.0"
                                % (a.workload, state_len, S, C, T, N),
                    "scan_mode": a.scan_mode, "seed": a.seed},
-        "roofline": roofline, "stages": stages, "cpu_baseline": cpu,
+        "roofline": roofline, "stages": stages, "fast_scan_mode": other, "cpu_baseline": cpu,
     }))
 
 
