@@ -182,11 +182,11 @@ struct __attribute__((aligned(16))) Elem {
     uint32_t info;  // state | prev << 16 | stay << 21
     float rest;     // score minus that guide term: what the next time step starts from
 };
-// mailbox of one step candidate (index 4i+b): its score, and the stay that claims it
+// mailbox of one step candidate (index 4i+b): what a stay that merged with it leaves behind
 struct __attribute__((aligned(16))) SlotRec {
     uint32_t tag;   // (t + 1) << 5 | stay element, written by the claiming stay at step t
-    float stay;     // that stay's score
-    float step;     // the step candidate's score, written by its own lane
+    float value;    // the step candidate's score after the merge
+    float step;     // the step candidate's own score (serial replay only)
     uint32_t pad;
 };
 
@@ -200,8 +200,23 @@ struct BeamShared {
     int consumed;          // rows the search wave is done with
 };
 
+// LDS of one chunk
 template <int S>
-__global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ scores,
+struct __attribute__((aligned(16))) BeamLds {
+    _Float16 row_s[BeamCfg<S>::kLdsRows][4 * S];
+    float row_b[BeamCfg<S>::kLdsRows][S];
+    BeamShared sh;
+    ofk_beam_slot_t trace[BeamCfg<S>::kTraceBlock][kW];
+    int32_t trace_state[BeamCfg<S>::kTraceBlock];
+    uint8_t trace_move[BeamCfg<S>::kTraceBlock];
+};
+
+// Two chunks per workgroup: a four-wave group gets one wave on each SIMD of its compute
+// unit, so every search wave has a SIMD to itself (two-wave groups share two SIMDs).
+constexpr int kGroupChunks = 2;
+
+template <int S>
+__global__ __launch_bounds__(128 * kGroupChunks) void beam_kernel(const _Float16 *__restrict__ scores,
                                                    const float *__restrict__ bwd,
                                                    ofk_beam_slot_t *__restrict__ beam,
                                                    int32_t *__restrict__ states, uint8_t *__restrict__ moves,
@@ -213,26 +228,31 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
     constexpr int RR = Cfg::kRegRows;
     constexpr int TB = Cfg::kTraceBlock;
 
-    __shared__ __attribute__((aligned(16))) _Float16 row_s[LR][4 * S];
-    __shared__ __attribute__((aligned(16))) float row_b[LR][S];
-    __shared__ __attribute__((aligned(16))) BeamShared sh;
-    __shared__ __attribute__((aligned(16))) ofk_beam_slot_t trace[TB][kW];
-    __shared__ int32_t trace_state[TB];
-    __shared__ uint8_t trace_move[TB];
+    __shared__ BeamLds<S> lds[kGroupChunks];
 
-    const int n = blockIdx.x;
+    // waves 0 .. kGroupChunks-1 search, the others load; wave k and wave k + kGroupChunks share a chunk
+    const int wave = (int)(threadIdx.x >> 6);
+    const int member = wave % kGroupChunks;
+    const int n = blockIdx.x * kGroupChunks + member;
     const int lane = threadIdx.x & 63;
+    auto &row_s = lds[member].row_s;
+    auto &row_b = lds[member].row_b;
+    BeamShared &sh = lds[member].sh;
+    auto &trace = lds[member].trace;
+    auto &trace_state = lds[member].trace_state;
+    auto &trace_move = lds[member].trace_move;
     const size_t row_stride = (size_t)N * 4 * S;
     const _Float16 *sc_n = scores + (size_t)n * 4 * S;
     const float *bw_n = bwd + (size_t)n * (size_t)(T + 1) * S;
 
-    if (threadIdx.x == 0) {
+    if (wave < kGroupChunks && lane == 0) {
         sh.ready = 0;
         sh.consumed = 0;
     }
     __syncthreads();
+    if (n >= N) return;  // odd batch: the last group has one chunk
 
-    if (threadIdx.x >= 64) {
+    if (wave >= kGroupChunks) {
         // ---- loader wave: row t = (scores[t], bwd[t+1]) into ring slot t % LR ----
         // The ring is spelled out as named registers (not an array indexed by a loop that
         // also contains the spin wait) so that every row stays in VGPRs.
@@ -366,8 +386,6 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
         const uint32_t h0 = crc2(hash, (uint32_t)b0);
         const uint32_t h1 = crc2(hash, (uint32_t)b0 + 1u);
         SlotRec *my_rec = &sh.rec[4 * i + b0];
-        my_rec[0].step = c0;
-        my_rec[1].step = c1;
 
         // which previous element j has hash_j == crc^-1(hash_i, last base of i)
         uint32_t match;
@@ -394,23 +412,36 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
         }
 
         // merge stays with the step spelling the same sequence (src/beam_search.c:281-316).
-        // The stay posts its score into the mailbox of the step it matches; then both
-        // sides read each other's score and apply their half of the merge.
+        // The stay's lane fetches the step's score from the lane that holds it, folds the two,
+        // keeps its half of the outcome and leaves the step's half in the step's mailbox.
         const bool mine = h == 0 && match != 0;
         if (ballot(mine) != 0) {
             const uint32_t now = (uint32_t)(t + 1);
             const uint32_t mytag = (now << 5) | (uint32_t)i;
-            const int target = 4 * (__builtin_ctz(match | 0x80000000u) & 31) + (state & 3);
-            if (mine) *reinterpret_cast<uint2 *>(&sh.rec[target]) = make_uint2(mytag, __float_as_uint(cs));
+            const int j = __builtin_ctz(match | 0x80000000u) & 31;
+            const int bi = state & 3;
+            const int holder = (j + ((bi & 2) << 4)) << 2;  // lane j + 32 * (bi >> 1), as a byte index
+            const float o0 = __int_as_float(__builtin_amdgcn_ds_bpermute(holder, __float_as_int(c0)));
+            const float o1 = __int_as_float(__builtin_amdgcn_ds_bpermute(holder, __float_as_int(c1)));
+            const float other = (bi & 1) ? o1 : o0;
+            const bool stay_wins = cs > other;
+            float folded = cs;
+            if (mine) folded = log_sum_exp(cs, other, sh.lse);
+            const int target = 4 * j + bi;
+            if (mine)
+                *reinterpret_cast<uint2 *>(&sh.rec[target]) =
+                    make_uint2(mytag, __float_as_uint(stay_wins ? -FLT_MAX : folded));
             wave_fence();
-            const uint4 claimed = mine ? *reinterpret_cast<const uint4 *>(&sh.rec[target]) : make_uint4(0, 0, 0, 0);
-            const uint4 box0 = *reinterpret_cast<const uint4 *>(&my_rec[0]);
-            const uint4 box1 = *reinterpret_cast<const uint4 *>(&my_rec[1]);
-            const bool odd = mine && ((match & (match - 1)) != 0 || claimed.x != mytag);
+            const uint32_t claimed = mine ? sh.rec[target].tag : mytag;
+            const uint2 box0 = *reinterpret_cast<const uint2 *>(&my_rec[0]);
+            const uint2 box1 = *reinterpret_cast<const uint2 *>(&my_rec[1]);
+            const bool odd = mine && ((match & (match - 1)) != 0 || claimed != mytag);
             if (ballot(odd) != 0 || (flags & 1)) {
                 // A stay with several equal hashes, or a step claimed by two stays (only
                 // possible after a CRC collision): replay the merges one by one in the
-                // CPU path's order.
+                // CPU path's order, from the scores as they were before any merge.
+                my_rec[0].step = c0;
+                my_rec[1].step = c1;
                 if (h == 0) sh.stay_score[i] = cs;
                 wave_fence();
                 if (lane == 0) {
@@ -420,12 +451,12 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
                         for (int b = 0; b < w; ++b) {
                             if (crc2(sh.hash[b], base) != ha) continue;
                             SlotRec *st = &sh.rec[4 * b + (int)base];
-                            const float folded = log_sum_exp(sh.stay_score[a], st->step, sh.lse);
+                            const float both = log_sum_exp(sh.stay_score[a], st->step, sh.lse);
                             if (sh.stay_score[a] > st->step) {
-                                sh.stay_score[a] = folded;
+                                sh.stay_score[a] = both;
                                 st->step = -FLT_MAX;
                             } else {
-                                st->step = folded;
+                                st->step = both;
                                 sh.stay_score[a] = -FLT_MAX;
                             }
                         }
@@ -436,36 +467,10 @@ __global__ __launch_bounds__(128) void beam_kernel(const _Float16 *__restrict__ 
                 c0 = my_rec[0].step;
                 c1 = my_rec[1].step;
             } else {
-                // Of every matched pair exactly one side survives and needs the folded
-                // score; the other becomes -FLT_MAX.  A lane rarely has more than one fold
-                // to compute (its stay, or one of its two steps), so the folds are taken
-                // one per lane and round, all lanes evaluating the polynomial together.
-                const float other = __uint_as_float(claimed.z);
-                const float st0 = __uint_as_float(box0.y), st1 = __uint_as_float(box1.y);
-                const bool hit0 = (box0.x >> 5) == now, hit1 = (box1.x >> 5) == now;
-                unsigned pend = 0;
-                if (mine) {
-                    if (cs > other) pend |= 1u; else cs = -FLT_MAX;
-                }
-                if (hit0) {
-                    if (st0 > c0) c0 = -FLT_MAX; else pend |= 2u;
-                }
-                if (hit1) {
-                    if (st1 > c1) c1 = -FLT_MAX; else pend |= 4u;
-                }
-                while (ballot(pend != 0) != 0) {
-                    // only the lanes that have a fold to do touch the coefficient table
-                    if (pend != 0) {
-                        const unsigned pick = pend & (0u - pend);
-                        const float x = pick == 1u ? cs : pick == 2u ? st0 : st1;
-                        const float y = pick == 1u ? other : pick == 2u ? c0 : c1;
-                        const float folded = log_sum_exp(x, y, sh.lse);
-                        if (pick == 1u) cs = folded;
-                        if (pick == 2u) c0 = folded;
-                        if (pick == 4u) c1 = folded;
-                        pend ^= pick;
-                    }
-                }
+                // of every matched pair one side carries the folded score on, the other is dropped
+                if (mine) cs = stay_wins ? folded : -FLT_MAX;
+                if ((box0.x >> 5) == now) c0 = __uint_as_float(box0.y);
+                if ((box1.x >> 5) == now) c1 = __uint_as_float(box1.y);
             }
         }
 
@@ -604,7 +609,7 @@ template <int S>
 int launch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                 uint8_t *moves, int T, int N, float log_cut, float stay, int flags, const double *lse_table,
                 hipStream_t st) {
-    hipLaunchKernelGGL((beam_kernel<S>), dim3(N), dim3(128), 0, st, static_cast<const _Float16 *>(scores),
+    hipLaunchKernelGGL((beam_kernel<S>), dim3((N + kGroupChunks - 1) / kGroupChunks), dim3(128 * kGroupChunks), 0, st, static_cast<const _Float16 *>(scores),
                        bwd, beam, states, moves, T, N, log_cut, stay, flags, lse_table);
     return (int)hipGetLastError();
 }
