@@ -76,12 +76,28 @@ __device__ __forceinline__ float lane_f(float x, int lane) {
 __device__ __forceinline__ uint32_t lane_u(uint32_t x, int lane) {
     return (uint32_t)__builtin_amdgcn_readlane((int)x, lane);
 }
+// Maximum over the wave, every lane active.  The rotate-and-max steps are single DPP
+// instructions written out by hand (the compiler's lowering of fmaxf after a DPP move
+// adds a move and a canonicalisation per step); each needs two idle cycles after the
+// instruction that wrote its source.  The last two steps carry the row maxima across
+// rows, so lane 63 ends up with the result.  The inputs are never NaN.
 __device__ __forceinline__ float wave_max(float x) {
-    x = fmaxf(x, dpp<0x128>(x));
-    x = fmaxf(x, dpp<0x124>(x));
-    x = fmaxf(x, dpp<0x122>(x));
-    x = fmaxf(x, dpp<0x121>(x));
-    return fmaxf(fmaxf(lane_f(x, 0), lane_f(x, 16)), fmaxf(lane_f(x, 32), lane_f(x, 48)));
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_ror:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(x));
+    return lane_f(x, 63);
 }
 __device__ __forceinline__ int wave_sum_i(int x) {
     x += __builtin_amdgcn_update_dpp(0, x, 0x128, 0xF, 0xF, true);
@@ -361,28 +377,46 @@ __global__ __launch_bounds__(128 * kGroupChunks) void beam_kernel(const _Float16
     // issue arbitration.
     __builtin_amdgcn_s_setprio(3);
     int rows_ready = 0;  // last value seen of the loader's counter; it is usually several rows ahead
-    for (int t = 0; t < T; ++t) {
-        while (rows_ready <= t) {
+    const int b0 = 2 * h;
+    // What a time step reads from LDS depends only on the beam it starts from, so it is
+    // fetched as soon as that beam is known (at the end of the previous step): the row
+    // entries of the lane's candidates and the 16 hashes this half of the wave compares with.
+    _Float16 r0h, r1h;
+    float2 g01;
+    float gst;
+    uint4 hq0, hq1, hq2, hq3;
+    auto fetch_row = [&](int tt) {
+        while (rows_ready <= tt) {
             rows_ready = observe(&sh.ready);
-            if (rows_ready <= t) __builtin_amdgcn_s_sleep(1);
+            if (rows_ready <= tt) __builtin_amdgcn_s_sleep(1);
         }
-        const int slot = t % LR;
+        const int slot = tt % LR;
         const _Float16 *rs = row_s[slot];
         const float *rb = row_b[slot];
-
+        const int lo4 = (state << 2) & (S - 1);
+        const int top = state >> (BITS - 2);
+        r0h = rs[4 * (lo4 + b0) + top];
+        r1h = rs[4 * (lo4 + b0 + 1) + top];
+        g01 = *reinterpret_cast<const float2 *>(&rb[lo4 + b0]);
+        gst = rb[state];
+        const uint4 *hp = reinterpret_cast<const uint4 *>(&sh.hash[16 * h]);
+        hq0 = hp[0];
+        hq1 = hp[1];
+        hq2 = hp[2];
+        hq3 = hp[3];
+    };
+    fetch_row(0);
+    for (int t = 0; t < T; ++t) {
         const bool valid = i < w;
         const uint64_t vm = ballot(valid);          // live elements, both halves
         const uint64_t vs = vm & 0xFFFFFFFFull;     // their stay candidates sit on lanes < 32
         const int lo4 = (state << 2) & (S - 1);
-        const int top = state >> (BITS - 2);
-        const int b0 = 2 * h;
-        const float r0 = (float)rs[4 * (lo4 + b0) + top];
-        const float r1 = (float)rs[4 * (lo4 + b0 + 1) + top];
-        const float2 g01 = *reinterpret_cast<const float2 *>(&rb[lo4 + b0]);
-        const float gst = rb[state];
+        const float r0 = (float)r0h;
+        const float r1 = (float)r1h;
         float c0 = (score + r0) + g01.x;
         float c1 = (score + r1) + g01.y;
         float cs = (score + stay) + gst;
+        publish(&sh.consumed, t + 1);  // everything this step needs of row t is in registers
         const uint32_t h0 = crc2(hash, (uint32_t)b0);
         const uint32_t h1 = crc2(hash, (uint32_t)b0 + 1u);
         SlotRec *my_rec = &sh.rec[4 * i + b0];
@@ -391,16 +425,17 @@ __global__ __launch_bounds__(128 * kGroupChunks) void beam_kernel(const _Float16
         uint32_t match;
         {
             const uint32_t want = crc2_inverse(hash, (uint32_t)state & 3u);
-            const uint4 *hp = reinterpret_cast<const uint4 *>(&sh.hash[16 * h]);
             uint32_t m = 0;
-#pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const uint4 x = hp[qd];
+            auto four = [&](const uint4 &x, int qd) {
                 m |= (x.x == want ? 1u : 0u) << (4 * qd);
                 m |= (x.y == want ? 1u : 0u) << (4 * qd + 1);
                 m |= (x.z == want ? 1u : 0u) << (4 * qd + 2);
                 m |= (x.w == want ? 1u : 0u) << (4 * qd + 3);
-            }
+            };
+            four(hq0, 0);
+            four(hq1, 1);
+            four(hq2, 2);
+            four(hq3, 3);
             m <<= 16 * h;
             {
                 // both halves of the wave looked at 16 hashes each: lanes i and i+32 join their masks
@@ -547,6 +582,7 @@ __global__ __launch_bounds__(128 * kGroupChunks) void beam_kernel(const _Float16
             info = 0;
         }
         state = (int)(info & 0xFFFFu);
+        if (t + 1 < T) fetch_row(t + 1);
 
         // last block: the best survivor goes to slot 0 (src/beam_search.c:398-414)
         if (t == T - 1) {
@@ -572,7 +608,6 @@ __global__ __launch_bounds__(128 * kGroupChunks) void beam_kernel(const _Float16
                 bv[(size_t)(t + 1) * kW + i] =
                     (ofk_beam_slot_t)((uint32_t)state | (((info >> 16) & 31u) << 10) | (((info >> 21) & 1u) << 15));
         }
-        publish(&sh.consumed, t + 1);
     }
 
     // ---- traceback from slot 0 of the last block (src/beam_search.c:432-439) ----
