@@ -315,14 +315,28 @@ static const ofk_phred_table_t *phred_for(ofa_gpubuf_t *g, const openfish_opt_t 
 
 /* ---- decode ---------------------------------------------------------------- */
 
-static void fetch_outputs(ofa_gpubuf_t *g, int T, int N, uint8_t **moves, char **sequence, char **qstring) {
+/* The three result buffers are the caller's to free (the reference's contract), so they are fresh
+ * allocations every call.  They are allocated and touched while the GPU works, which takes the page
+ * faults off the path between the last kernel and the return. */
+/* all three results over the main stream (the stage-level entry point) */
+static void fetch_outputs(ofa_gpubuf_t *g, int T, int N, uint8_t **moves, char **sequence, char **qstring);
+
+static void alloc_outputs(int T, int N, uint8_t **moves, char **sequence, char **qstring) {
     const size_t nt = (size_t)N * (size_t)T;
     *moves = (uint8_t *)host_alloc(nt);
     *sequence = (char *)host_alloc(nt);
     *qstring = (char *)host_alloc(nt);
+    memset(*moves, 0, nt);
+    memset(*sequence, 0, nt);
+    memset(*qstring, 0, nt);
+}
+
+static void fetch_outputs(ofa_gpubuf_t *g, int T, int N, uint8_t **moves, char **sequence, char **qstring) {
+    const size_t nt = (size_t)N * (size_t)T;
     HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_main));
     HIP_OK(hipMemcpyAsync(g->h_out + nt, g->pub.sequence, nt, hipMemcpyDeviceToHost, g->s_main));
     HIP_OK(hipMemcpyAsync(g->h_out + 2 * nt, g->pub.qstring, nt, hipMemcpyDeviceToHost, g->s_main));
+    alloc_outputs(T, N, moves, sequence, qstring);
     HIP_OK(hipStreamSynchronize(g->s_main));
     memcpy(*moves, g->h_out, nt);
     memcpy(*sequence, g->h_out + nt, nt);
@@ -341,6 +355,7 @@ void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC
     check_scores_any(T, N, C, scores_TNC, state_len, options, 1);
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     const float stay = options->blank_score; /* as the reference GPU path, src/decode_hip.hip:120 */
+    const size_t nt = (size_t)N * (size_t)T;
     OPENFISH_LOG_TRACE("scores tensor dim: %d, %d, %d", T, N, C);
 
     join_null_stream(g);
@@ -355,6 +370,8 @@ void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC
                               (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, log_beam_cut(options),
                               stay, g->lse_table, g->s_side), "beam_search");
     HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_side));
+    /* the moves are final once the beam search is: they travel while the sequence stage runs */
+    HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_side));
 
     launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->s_main),
               "fwd_post_scan");
@@ -366,8 +383,15 @@ void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC
                            g->pub.base_probs, g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N,
                            state_len, phred_for(g, options), g->s_main), "sequence");
     HIP_OK(hipEventRecord(g->ev[EV_SEQ_END], g->s_main));
+    HIP_OK(hipMemcpyAsync(g->h_out + nt, g->pub.sequence, nt, hipMemcpyDeviceToHost, g->s_main));
+    HIP_OK(hipMemcpyAsync(g->h_out + 2 * nt, g->pub.qstring, nt, hipMemcpyDeviceToHost, g->s_main));
 
-    fetch_outputs(g, T, N, moves, sequence, qstring);
+    alloc_outputs(T, N, moves, sequence, qstring);
+    HIP_OK(hipStreamSynchronize(g->s_side));
+    memcpy(*moves, g->h_out, nt);
+    HIP_OK(hipStreamSynchronize(g->s_main));
+    memcpy(*sequence, g->h_out + nt, nt);
+    memcpy(*qstring, g->h_out + 2 * nt, nt);
     g->timed = 1;
 }
 
