@@ -227,12 +227,13 @@ struct __attribute__((aligned(16))) BeamLds {
     uint8_t trace_move[BeamCfg<S>::kTraceBlock];
 };
 
-// Two chunks per workgroup: a four-wave group gets one wave on each SIMD of its compute
-// unit, so every search wave has a SIMD to itself (two-wave groups share two SIMDs).
-constexpr int kGroupChunks = 2;
-
-template <int S>
-__global__ __launch_bounds__(128 * kGroupChunks) void beam_kernel(const _Float16 *__restrict__ scores,
+// CPG chunks per workgroup.  The waves of a group are dealt round over the four SIMDs of
+// its compute unit (wave k and wave k + 4 share one), while two-wave groups were measured
+// to pile onto two SIMDs.  With two chunks a group is four waves, two of them searching;
+// with four chunks it is eight waves and every SIMD holds exactly one search wave and one
+// loader, which is what a batch of more than two chunks per compute unit needs.
+template <int S, int CPG>
+__global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restrict__ scores,
                                                    const float *__restrict__ bwd,
                                                    ofk_beam_slot_t *__restrict__ beam,
                                                    int32_t *__restrict__ states, uint8_t *__restrict__ moves,
@@ -244,6 +245,7 @@ __global__ __launch_bounds__(128 * kGroupChunks) void beam_kernel(const _Float16
     constexpr int RR = Cfg::kRegRows;
     constexpr int TB = Cfg::kTraceBlock;
 
+    constexpr int kGroupChunks = CPG;
     __shared__ BeamLds<S> lds[kGroupChunks];
 
     // waves 0 .. kGroupChunks-1 search, the others load; wave k and wave k + kGroupChunks share a chunk
@@ -644,8 +646,19 @@ template <int S>
 int launch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                 uint8_t *moves, int T, int N, float log_cut, float stay, int flags, const double *lse_table,
                 hipStream_t st) {
-    hipLaunchKernelGGL((beam_kernel<S>), dim3((N + kGroupChunks - 1) / kGroupChunks), dim3(128 * kGroupChunks), 0, st, static_cast<const _Float16 *>(scores),
-                       bwd, beam, states, moves, T, N, log_cut, stay, flags, lse_table);
+    // 256 compute units: up to 512 chunks fit two to a unit; larger batches go four to a group
+    // where the LDS of four chunks fits (64 and 256 states)
+    if constexpr (S <= 256) {
+        if (N > 512) {
+            hipLaunchKernelGGL((beam_kernel<S, 4>), dim3((N + 3) / 4), dim3(512), 0, st,
+                               static_cast<const _Float16 *>(scores), bwd, beam, states, moves, T, N, log_cut,
+                               stay, flags, lse_table);
+            return (int)hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((beam_kernel<S, 2>), dim3((N + 1) / 2), dim3(256), 0, st,
+                           static_cast<const _Float16 *>(scores), bwd, beam, states, moves, T, N, log_cut, stay,
+                           flags, lse_table);
     return (int)hipGetLastError();
 }
 

@@ -364,20 +364,24 @@ void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC
     launch_ok(ofk_bwd_scan(scores_TNC, g->pub.bwd_NTC, T, N, state_len, stay, g->s_main), "bwd_scan");
     HIP_OK(hipEventRecord(g->ev[EV_BWD_END], g->s_main));
 
-    HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BWD_END], 0));
-    HIP_OK(hipEventRecord(g->ev[EV_BEAM_START], g->s_side));
+    /* The beam search is the longer of the two stages that follow and wants its workgroups (large
+     * LDS blocks) resident before the forward sweep fills the compute units: it stays on the stream
+     * the backward sweep ran on and so starts first; the forward sweep follows through an event. */
+    HIP_OK(hipEventRecord(g->ev[EV_BEAM_START], g->s_main));
     launch_ok(ofk_beam_search(scores_TNC, g->pub.bwd_NTC, (ofk_beam_slot_t *)g->pub.beam_vector,
                               (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, log_beam_cut(options),
-                              stay, g->lse_table, g->s_side), "beam_search");
-    HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_side));
+                              stay, g->lse_table, g->s_main), "beam_search");
+    HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_main));
+
+    HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BWD_END], 0));
+    launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->s_side),
+              "fwd_post_scan");
+    HIP_OK(hipEventRecord(g->ev[EV_FWD_END], g->s_side));
     /* the moves are final once the beam search is: they travel while the sequence stage runs */
+    HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BEAM_END], 0));
     HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_side));
 
-    launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->s_main),
-              "fwd_post_scan");
-    HIP_OK(hipEventRecord(g->ev[EV_FWD_END], g->s_main));
-
-    HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_BEAM_END], 0));
+    HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_FWD_END], 0));
     HIP_OK(hipEventRecord(g->ev[EV_SEQ_START], g->s_main));
     launch_ok(ofk_sequence(g->pub.post_NTC, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data,
                            g->pub.base_probs, g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N,

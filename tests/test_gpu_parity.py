@@ -129,6 +129,8 @@ SHAPES = [
     (3, 1, 1, False), (3, 2, 3, False), (3, 7, 5, False), (3, 9, 4, True), (3, 333, 13, True),
     (4, 1, 2, False), (4, 5, 1, False), (4, 257, 9, False), (4, 130, 6, True),
     (5, 3, 1, False), (5, 61, 3, False), (5, 40, 2, True),
+    # more than 512 chunks: the beam search runs four chunks to a workgroup, the last group ragged
+    (3, 24, 517, False), (4, 12, 514, True),
 ]
 
 
