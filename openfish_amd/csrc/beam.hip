@@ -427,17 +427,29 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         uint32_t match;
         {
             const uint32_t want = crc2_inverse(hash, (uint32_t)state & 3u);
+            // Bit k of m says whether hash k of this half equals `want`.  Each comparison is
+            // shifted in with an add-with-carry (m = 2m + equal), two instructions per hash; the
+            // four comparisons of a vector are issued before the four adds so that no add reads
+            // a comparison result sooner than three instructions after it was written.
             uint32_t m = 0;
-            auto four = [&](const uint4 &x, int qd) {
-                m |= (x.x == want ? 1u : 0u) << (4 * qd);
-                m |= (x.y == want ? 1u : 0u) << (4 * qd + 1);
-                m |= (x.z == want ? 1u : 0u) << (4 * qd + 2);
-                m |= (x.w == want ? 1u : 0u) << (4 * qd + 3);
+            auto four = [&](const uint4 &x) {
+                uint64_t e0, e1, e2, e3, carry;
+                asm("v_cmp_eq_u32_e64 %[e3], %[w], %[x3]\n\t"
+                    "v_cmp_eq_u32_e64 %[e2], %[w], %[x2]\n\t"
+                    "v_cmp_eq_u32_e64 %[e1], %[w], %[x1]\n\t"
+                    "v_cmp_eq_u32_e64 %[e0], %[w], %[x0]\n\t"
+                    "v_addc_co_u32_e64 %[m], %[c], %[m], %[m], %[e3]\n\t"
+                    "v_addc_co_u32_e64 %[m], %[c], %[m], %[m], %[e2]\n\t"
+                    "v_addc_co_u32_e64 %[m], %[c], %[m], %[m], %[e1]\n\t"
+                    "v_addc_co_u32_e64 %[m], %[c], %[m], %[m], %[e0]"
+                    : [m] "+v"(m), [e0] "=&s"(e0), [e1] "=&s"(e1), [e2] "=&s"(e2), [e3] "=&s"(e3),
+                      [c] "=&s"(carry)
+                    : [w] "v"(want), [x0] "v"(x.x), [x1] "v"(x.y), [x2] "v"(x.z), [x3] "v"(x.w));
             };
-            four(hq0, 0);
-            four(hq1, 1);
-            four(hq2, 2);
-            four(hq3, 3);
+            four(hq3);
+            four(hq2);
+            four(hq1);
+            four(hq0);
             m <<= 16 * h;
             {
                 // both halves of the wave looked at 16 hashes each: lanes i and i+32 join their masks
@@ -469,9 +481,12 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 *reinterpret_cast<uint2 *>(&sh.rec[target]) =
                     make_uint2(mytag, __float_as_uint(stay_wins ? -FLT_MAX : folded));
             wave_fence();
-            const uint32_t claimed = mine ? sh.rec[target].tag : mytag;
-            const uint2 box0 = *reinterpret_cast<const uint2 *>(&my_rec[0]);
-            const uint2 box1 = *reinterpret_cast<const uint2 *>(&my_rec[1]);
+            uint32_t claimed = mine ? sh.rec[target].tag : mytag;
+            uint2 box0 = *reinterpret_cast<const uint2 *>(&my_rec[0]);
+            uint2 box1 = *reinterpret_cast<const uint2 *>(&my_rec[1]);
+            // keep the three reads together in one LDS round trip (the compiler would otherwise
+            // sink the mailbox reads below the branch that follows)
+            asm volatile("" : "+v"(claimed), "+v"(box0.x), "+v"(box0.y), "+v"(box1.x), "+v"(box1.y));
             const bool odd = mine && ((match & (match - 1)) != 0 || claimed != mytag);
             if (ballot(odd) != 0 || (flags & 1)) {
                 // A stay with several equal hashes, or a step claimed by two stays (only

@@ -43,13 +43,13 @@ def test_exp_relative_error_below_2_pow_minus_46(lib):
     rng = np.random.default_rng(1)
     d = np.concatenate([-80 * rng.random(400000), -rng.random(200000), -1e-3 * rng.random(100000),
                         -(np.arange(0, 2560) / 32.0), [0.0, -0.0, -1e-30, -79.99999]]).astype(np.float32)
-    assert lib.max_rel_err_exp(fptr(d), d.size) < 2.0 ** -46
+    assert lib.max_rel_err_exp(fptr(d), d.size) < 2.0 ** -50
 
 
 def test_ldexp_scaled_exp_and_table_log(lib):
     rng = np.random.default_rng(4)
     d = np.concatenate([-100 * rng.random(400000), -rng.random(100000), [0.0, -700.0]]).astype(np.float32)
-    assert lib.max_rel_err_exp_ldexp(fptr(d), d.size) < 2.0 ** -46
+    assert lib.max_rel_err_exp_ldexp(fptr(d), d.size) < 2.0 ** -50
     far = np.array([-745.0, -20000.0, -1e8], np.float32)  # subnormal or zero results: absolute check
     assert lib.max_rel_err_exp_ldexp(fptr(far[1:]), 2) == 0.0  # exactly zero, like exp()
     s = np.concatenate([1 + 4 * rng.random(500000), 1 + 1e-4 * rng.random(100000),
