@@ -527,9 +527,12 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         }
 
         // cut-off (src/beam_search.c:320-381)
-        float best = -FLT_MAX;
-        if (valid) best = fmaxf(c0, c1);
-        if (valid && h == 0) best = fmaxf(best, cs);
+        // dead lanes carry -FLT_MAX as their score, so their candidates are about -FLT_MAX too
+        float best;
+        {
+            const float cs_or_none = h == 0 ? cs : -FLT_MAX;
+            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(best) : "v"(c0), "v"(c1), "v"(cs_or_none));
+        }
         best = wave_max(best);
 
         float cut = best - log_cut;
@@ -567,7 +570,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const int before = popc64(k0 & below) + popc64(k1 & below);
             const uint32_t k0lo = (uint32_t)k0, k1lo = (uint32_t)k1;
             const int same = h == 0 ? 0 : (int)((k0lo >> i) & 1u) + (int)((k1lo >> i) & 1u);
-            const bool keep0 = (k0 >> lane) & 1u, keep1 = (k1 >> lane) & 1u, keeps = (ks >> lane) & 1u;
+            const bool keep0 = valid && c0 >= cut, keep1 = valid && c1 >= cut;  // this lane's bits of k0, k1
+            const bool keeps = valid && h == 0 && cs >= cut;                      // and of ks
             const int rank0 = before + same;
             const int rank1 = rank0 + (keep0 ? 1 : 0);
             const int ranks = popc64(k0) + popc64(k1) + popc64(ks & below);
@@ -587,7 +591,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             wave_fence();
         }
         w = kept;
-        float rest = 0.f;
+        float rest = -FLT_MAX;
         if (i < w) {
             const Elem e = sh.elem[i];
             hash = e.hash;
@@ -595,7 +599,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             info = e.info;
             rest = e.rest;
         } else {
-            score = 0.f;
+            score = -FLT_MAX;
             info = 0;
         }
         state = (int)(info & 0xFFFFu);
