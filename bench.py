@@ -130,7 +130,7 @@ def main():
     ap.add_argument("--workload", default="hac", choices=sorted(WORKLOADS) + ["rotary"])
     ap.add_argument("--chunks", type=int, default=0, help="override N")
     ap.add_argument("--scan-mode", default="precise", choices=("precise", "fast"))
-    ap.add_argument("--cpu-sample", type=int, default=64, help="chunks timed on the CPU path (0 = skip)")
+    ap.add_argument("--cpu-sample", type=int, default=512, help="chunks timed on the CPU path (0 = skip; capped at N)")
     ap.add_argument("--seed", type=int, default=20251125)
     ap.add_argument("--alt-steps", type=int, default=3,
                     help="extra timed calls with the hardware-exp scan arithmetic, reported beside the main result (0 = skip)")
