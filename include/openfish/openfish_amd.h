@@ -90,6 +90,28 @@ void openfish_amd_decode_from_tensors(int T, int N, int C, const void *scores, i
                                       const float *post, const openfish_gpubuf_t *gpubuf,
                                       uint8_t **moves, char **sequence, char **qstring);
 
+/*
+ * openfish_decode_gpu in two halves, for a caller that keeps more than one batch in
+ * flight from one thread (one gpubuf per batch in flight).  The blocking call of the
+ * reference (src/openfish.c:43-63, src/decode_hip.hip:83-217: five device
+ * synchronisations and three host allocations per call) is enqueue + wait + a copy
+ * into fresh malloc'd buffers.
+ *
+ * openfish_amd_decode_enqueue queues every kernel and the copies of the results into
+ * the gpubuf's pinned host buffer, ordered after work already queued on the null
+ * stream, and returns without waiting.  The scores must stay valid and unchanged until
+ * the wait returns.  A gpubuf holds one enqueued decode at a time.
+ *
+ * openfish_amd_decode_wait blocks until that decode is complete and hands out pointers
+ * into the pinned buffer: N*T bytes each, chunk n at n*T, as openfish_decode_gpu lays
+ * them out.  They stay valid until the next enqueue (or decode) on the same gpubuf and
+ * belong to the gpubuf: the caller does not free them.
+ */
+void openfish_amd_decode_enqueue(int T, int N, int C, const void *scores_TNC, int state_len,
+                                 const openfish_opt_t *options, const openfish_gpubuf_t *gpubuf);
+void openfish_amd_decode_wait(const openfish_gpubuf_t *gpubuf, const uint8_t **moves,
+                              const char **sequence, const char **qstring);
+
 /* ---- measurement ---- */
 
 enum openfish_amd_stage {

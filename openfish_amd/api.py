@@ -77,6 +77,8 @@ _SIGS = {
     "openfish_amd_fwd_post_scan": (None, [_i, _i, _i, _vp, _i, _f, _vp, _vp]),
     "openfish_amd_beam_search": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _bufp]),
     "openfish_amd_sequence": (None, [_i, _i, _i, _optp, _vp, _bufp]),
+    "openfish_amd_decode_enqueue": (None, [_i, _i, _i, _vp, _i, _optp, _bufp]),
+    "openfish_amd_decode_wait": (None, [_bufp, _pp, _pp, _pp]),
     "openfish_amd_decode_from_tensors": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _vp, _bufp, _pp, _pp, _pp]),
     "openfish_amd_last_timings": (_i, [_bufp, C.POINTER(C.c_float), _i]),
     "openfish_amd_set_debug_flags": (None, [_i]),
@@ -201,6 +203,25 @@ def openfish_decode_gpu(T, N, Cc, scores_dev, state_len, options, gpubuf):
     _L.openfish_decode_gpu(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), gpubuf.handle,
                            C.byref(mv), C.byref(sq), C.byref(qs))
     return _take(mv, N, T), _take(sq, N, T), _take(qs, N, T)
+
+
+def openfish_amd_decode_enqueue(T, N, Cc, scores_dev, state_len, options, gpubuf):
+    """queue one decode on the gpubuf and return at once; scores_dev must stay alive until the wait"""
+    _L.openfish_amd_decode_enqueue(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), gpubuf.handle)
+    gpubuf._pending_shape = (N, T)
+
+
+def openfish_amd_decode_wait(gpubuf):
+    """(moves, sequence, qstring) of the enqueued decode as uint8 [N, T] arrays (copies of the
+    library's pinned buffer)"""
+    N, T = gpubuf._pending_shape
+    mv, sq, qs = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    _L.openfish_amd_decode_wait(gpubuf.handle, C.byref(mv), C.byref(sq), C.byref(qs))
+    out = []
+    for p in (mv, sq, qs):
+        buf = (C.c_uint8 * (N * T)).from_address(p.value)
+        out.append(np.frombuffer(buf, np.uint8).reshape(N, T).copy())
+    return tuple(out)
 
 
 def openfish_amd_decode_from_tensors(T, N, Cc, scores_dev, state_len, options, bwd_dev, post_dev, gpubuf):

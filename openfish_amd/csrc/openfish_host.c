@@ -131,6 +131,8 @@ typedef struct {
     hipEvent_t ev[EV_COUNT];
     float ms[OPENFISH_AMD_STAGE_COUNT];
     int timed;
+    int pending;           /* a decode has been enqueued and not yet waited for */
+    int pend_T, pend_N;    /* its shape */
     ofk_phred_table_t phred; /* thresholds for (phred_shift, phred_scale) */
     float phred_shift, phred_scale;
     int phred_valid;
@@ -349,18 +351,17 @@ static void join_null_stream(ofa_gpubuf_t *g) {
     HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_JOIN], 0));
 }
 
-void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC, const int state_len,
-                         const openfish_opt_t *options, const openfish_gpubuf_t *gpubuf, uint8_t **moves,
-                         char **sequence, char **qstring) {
-    check_scores_any(T, N, C, scores_TNC, state_len, options, 1);
-    ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
+/* Queue one decode on the gpubuf's streams, results into its pinned staging buffer; returns
+ * without waiting for the GPU. */
+static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int C, const void *scores_TNC,
+                           const int state_len, const openfish_opt_t *options) {
     const float stay = options->blank_score; /* as the reference GPU path, src/decode_hip.hip:120 */
     const size_t nt = (size_t)N * (size_t)T;
-    OPENFISH_LOG_TRACE("scores tensor dim: %d, %d, %d", T, N, C);
+    if (g->pending) die("this gpubuf already holds a decode that has not been waited for");
 
     join_null_stream(g);
     HIP_OK(hipEventRecord(g->ev[EV_START], g->s_main));
-    scores_TNC = (void *)four_columns(g, T, N, C, scores_TNC, state_len);
+    scores_TNC = four_columns(g, T, N, C, scores_TNC, state_len);
     launch_ok(ofk_bwd_scan(scores_TNC, g->pub.bwd_NTC, T, N, state_len, stay, g->s_main), "bwd_scan");
     HIP_OK(hipEventRecord(g->ev[EV_BWD_END], g->s_main));
 
@@ -389,13 +390,50 @@ void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC
     HIP_OK(hipEventRecord(g->ev[EV_SEQ_END], g->s_main));
     HIP_OK(hipMemcpyAsync(g->h_out + nt, g->pub.sequence, nt, hipMemcpyDeviceToHost, g->s_main));
     HIP_OK(hipMemcpyAsync(g->h_out + 2 * nt, g->pub.qstring, nt, hipMemcpyDeviceToHost, g->s_main));
+    g->pending = 1;
+    g->pend_T = T;
+    g->pend_N = N;
+}
 
+void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC, const int state_len,
+                         const openfish_opt_t *options, const openfish_gpubuf_t *gpubuf, uint8_t **moves,
+                         char **sequence, char **qstring) {
+    check_scores_any(T, N, C, scores_TNC, state_len, options, 1);
+    ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
+    const size_t nt = (size_t)N * (size_t)T;
+    OPENFISH_LOG_TRACE("scores tensor dim: %d, %d, %d", T, N, C);
+
+    enqueue_decode(g, T, N, C, scores_TNC, state_len, options);
     alloc_outputs(T, N, moves, sequence, qstring);
     HIP_OK(hipStreamSynchronize(g->s_side));
     memcpy(*moves, g->h_out, nt);
     HIP_OK(hipStreamSynchronize(g->s_main));
     memcpy(*sequence, g->h_out + nt, nt);
     memcpy(*qstring, g->h_out + 2 * nt, nt);
+    g->pending = 0;
+    g->timed = 1;
+}
+
+void openfish_amd_decode_enqueue(int T, int N, int C, const void *scores_TNC, int state_len,
+                                 const openfish_opt_t *options, const openfish_gpubuf_t *gpubuf) {
+    check_scores_any(T, N, C, scores_TNC, state_len, options, 1);
+    ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
+    enqueue_decode(g, T, N, C, scores_TNC, state_len, options);
+}
+
+void openfish_amd_decode_wait(const openfish_gpubuf_t *gpubuf, const uint8_t **moves, const char **sequence,
+                              const char **qstring) {
+    ofa_gpubuf_t *g = (ofa_gpubuf_t *)gpubuf;
+    if (!g || g->magic != OFA_MAGIC) die("gpubuf was not created by openfish_gpubuf_init");
+    if (!g->pending) die("decode_wait: nothing was enqueued on this gpubuf");
+    if (!moves || !sequence || !qstring) die("decode_wait: output pointer is NULL");
+    const size_t nt = (size_t)g->pend_N * (size_t)g->pend_T;
+    HIP_OK(hipStreamSynchronize(g->s_side));
+    HIP_OK(hipStreamSynchronize(g->s_main));
+    *moves = g->h_out;
+    *sequence = (const char *)g->h_out + nt;
+    *qstring = (const char *)g->h_out + 2 * nt;
+    g->pending = 0;
     g->timed = 1;
 }
 

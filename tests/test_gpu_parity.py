@@ -199,6 +199,27 @@ def test_gpubuf_is_reusable_for_smaller_batches(api):
         assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
 
 
+def test_enqueue_and_wait_with_two_batches_in_flight(api):
+    """two gpubufs, both decodes queued before either is waited for, twice over; results as
+    the oracle's (and so as the blocking call's)"""
+    kw = dict(q_scale=0.95, q_shift=-0.2)
+    opt = api.DECODER_INIT(**kw)
+    shapes = ((4, 300, 7), (3, 420, 9))
+    bufs = [api.GpuBuf(T, N, sl) for sl, T, N in shapes]
+    for rnd in range(2):
+        inputs = [synth.crf_scores(T, N, sl, seed=600 + 10 * rnd + k) for k, (sl, T, N) in enumerate(shapes)]
+        dev = [api.upload_scores_to_hip(x) for x in inputs]
+        for (sl, T, N), sc, gb in zip(shapes, dev, bufs):
+            api.openfish_amd_decode_enqueue(T, N, 4 * 4 ** sl, sc, sl, opt, gb)
+        for (sl, T, N), x, gb in zip(shapes, inputs, bufs):
+            mv, sq, qs = api.openfish_amd_decode_wait(gb)
+            ref = O.decode(x.astype(np.float32), sl, kw, nthreads=4)
+            assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"])
+            assert np.array_equal(qs, ref["qstring"])
+            assert set(gb.timings()) >= {"bwd", "beam"}
+        del dev
+
+
 @pytest.mark.parametrize("state_len,T,N", [(3, 150, 5), (4, 90, 3), (5, 40, 2)])
 def test_five_column_input_equals_its_four_column_view(api, state_len, T, N):
     """C = 5*S: a blank column in front of the four step columns of every state"""
