@@ -1,12 +1,13 @@
-// Beam search over one chunk per workgroup, gfx950.
+// Beam search over CRF scores, gfx950.
 //
-// A workgroup is two wavefronts.  Wave 1 streams the rows the search needs
-// (scores[t] as fp16 and bwd[t+1] as fp32) from HBM into an LDS ring, several
-// rows ahead; wave 0 runs the search with the 32-wide beam resident in
-// registers/LDS.  The two communicate through two LDS counters (rows ready /
-// rows consumed), so the search never waits on a dependent HBM gather.
+// Every chunk is served by two wavefronts of a workgroup.  The loader wave streams the
+// rows the search needs (scores[t] as fp16 and bwd[t+1] as fp32) from HBM into an LDS
+// ring, several rows ahead; the search wave runs the search with the 32-wide beam
+// resident in registers/LDS.  The two communicate through two LDS counters (rows ready /
+// rows consumed), so the search never waits on a dependent HBM gather.  A workgroup holds
+// two or four chunks, so that its waves spread over the four SIMDs of a compute unit.
 //
-// Wave 0 lane layout: lane = i + 32*h holds beam element i (mirrored in both
+// Search wave lane layout: lane = i + 32*h holds beam element i (mirrored in both
 // halves) and the step candidates with new base 2h and 2h+1; lanes < 32 also hold
 // the stay candidate.  Candidate order is the CPU path's: steps 4i+b, then stays.
 // The search reproduces the CPU path (reference src/beam_search.c:117-439) to the
@@ -284,7 +285,9 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         };
         auto hand_over = [&](RowRegs<8 * S> &rs, RowRegs<4 * S> &rb, int t) {
             if (t < T) {
-                while (t - observe(&sh.consumed) >= LR) __builtin_amdgcn_s_sleep(1);
+                // the ring is full most of the time (a search step takes about 3000 cycles): poll
+                // seldom, the rows in registers and in the ring leave ample slack for waking up late
+                while (t - observe(&sh.consumed) >= LR) __builtin_amdgcn_s_sleep(8);
                 const int slot = t % LR;
                 rs.store(reinterpret_cast<char *>(row_s[slot]), lane);
                 rb.store(reinterpret_cast<char *>(row_b[slot]), lane);
