@@ -13,6 +13,8 @@
 extern "C" {
 #endif
 
+/* longest chunk in time steps: the sequence stage keeps 14 bytes per step in LDS (160 KB) */
+#define OFK_MAX_T 8192
 #define OFK_BAD_ARGS (-1)
 #define OFK_BEAM_WIDTH 32
 

@@ -149,6 +149,7 @@ static void check_state_len(int state_len) {
 openfish_gpubuf_t *openfish_gpubuf_init(const int T, const int N, const int state_len) {
     check_state_len(state_len);
     if (T < 1 || N < 1) die("gpubuf: T and N must be positive");
+    if (T > OFK_MAX_T) die("gpubuf: chunks longer than 8192 time steps are not supported");
     const size_t S = (size_t)states_of(state_len), nt = (size_t)N * (size_t)T;
     const size_t tens = sizeof(float) * (size_t)N * (size_t)(T + 1) * S;
     ofa_gpubuf_t *g = (ofa_gpubuf_t *)host_alloc(sizeof *g);
@@ -216,6 +217,7 @@ static void check_scores_any(int T, int N, int C, const void *scores, int state_
                              int allow_blank_column) {
     check_state_len(state_len);
     if (T < 1 || N < 1) die("T and N must be positive");
+    if (T > OFK_MAX_T) die("chunks longer than 8192 time steps are not supported");
     if (C != 4 * states_of(state_len) && !(allow_blank_column && C == 5 * states_of(state_len)))
         die("C must be 4 * 4^state_len (one score per state and dropped base)");
     if (!scores) die("scores_TNC is NULL");

@@ -137,6 +137,11 @@ int launch_sequence(const float *post, int32_t *states, const uint8_t *moves, fl
                     float *base_probs, float *total_probs, char *sequence, char *qstring, int T, int N,
                     const ofk_phred_table_t &phred, hipStream_t st) {
     const size_t lds = (size_t)T * (4 + 4 + 1 + 1) + (size_t)(T + 1) * 4;
+    if (lds > 64 * 1024) {  // beyond the default limit of dynamic LDS; the compute unit has 160 KB
+        const hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(&sequence_kernel<S>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (rc != hipSuccess) return (int)rc;
+    }
     hipLaunchKernelGGL((sequence_kernel<S>), dim3(N), dim3(kThreads), lds, st, post, states, moves, qual_data,
                        base_probs, total_probs, sequence, qstring, T, phred);
     return (int)hipGetLastError();
@@ -147,9 +152,9 @@ int launch_sequence(const float *post, int32_t *states, const uint8_t *moves, fl
 extern "C" int ofk_sequence(const float *post, int32_t *states, const uint8_t *moves, float *qual_data,
                             float *base_probs, float *total_probs, char *sequence, char *qstring, int T, int N,
                             int state_len, const ofk_phred_table_t *phred, void *stream) {
-    // the per-chunk tables live in LDS: 14 bytes per time step, at most 64 KB
+    // the per-chunk tables live in LDS: 14 bytes per time step
     if (!post || !states || !moves || !qual_data || !base_probs || !total_probs || !sequence || !qstring ||
-        !phred || T < 1 || T > 4096 || N < 1)
+        !phred || T < 1 || T > OFK_MAX_T || N < 1)
         return OFK_BAD_ARGS;
     if (reinterpret_cast<uintptr_t>(qual_data) & 15u) return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);

@@ -131,6 +131,8 @@ SHAPES = [
     (5, 3, 1, False), (5, 61, 3, False), (5, 40, 2, True),
     # more than 512 chunks: the beam search runs four chunks to a workgroup, the last group ragged
     (3, 24, 517, False), (4, 12, 514, True),
+    # long chunks: the sequence stage's per-chunk tables beyond 64 KB of LDS, and the longest allowed
+    (3, 4700, 2, False), (4, 8192, 1, False),
 ]
 
 
