@@ -165,21 +165,6 @@ def main():
     scores = api.upload_scores_to_hip(s16)
     gpubuf = api.GpuBuf(T, N, state_len)
 
-    # what a plain streaming copy kernel reaches on this device (1 GiB each way, read + write
-    # counted), as a second yardstick beside the published 8 TB/s; with --calibrate-copy the
-    # same kernel runs once more for the counter calibration of the profiles
-    copy_gbs = None
-    if a.copy_mib > 0:
-        nbytes = a.copy_mib << 20
-        src, dst = api.DeviceBuffer(nbytes), api.DeviceBuffer(nbytes)
-        src.fill(1)
-        api.lib().openfish_amd_copy(dst.ptr, src.ptr, nbytes)
-        tc = time.perf_counter()
-        for _ in range(5):
-            api.lib().openfish_amd_copy(dst.ptr, src.ptr, nbytes)
-        copy_gbs = 5 * 2 * nbytes / 1e9 / (time.perf_counter() - tc)
-        src.free()
-        dst.free()
     if a.calibrate_copy:
         nbytes = a.calibrate_copy << 20
         src, dst = api.DeviceBuffer(nbytes), api.DeviceBuffer(nbytes)
@@ -212,9 +197,6 @@ def main():
     scan_gbs = (need["bwd"] + need["fwd_post"]) / 1e9 / (scan_ms / 1e3)
     stages["scan_plus_posterior"] = {"ms": round(scan_ms, 4), "GBps": round(scan_gbs, 1),
                                      "frac_of_hbm_peak": round(scan_gbs / HBM_PEAK_GBS, 4)}
-    if copy_gbs:
-        stages["device_copy_GBps"] = round(copy_gbs, 1)
-        stages["scan_plus_posterior"]["frac_of_device_copy"] = round(scan_gbs / copy_gbs, 4)
     dominant = max(("bwd", "fwd_post", "beam", "sequence"), key=lambda k: stages[k]["ms"])
     traffic = MEASURED_TRAFFIC_GB.get((a.workload, N, dominant))
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
@@ -257,6 +239,26 @@ def main():
                    "calls": 2 * a.overlap_steps,
                    "note": "one thread, openfish_amd_decode_enqueue/_wait alternating over two gpubufs; "
                            "not `value`"}
+
+    # what a plain streaming copy kernel reaches on this device (1 GiB each way, read + write
+    # counted), as a second yardstick beside the published 8 TB/s.  Measured after the timed loops:
+    # allocating and freeing the two large buffers first was seen to add 0.2 ms of host time to
+    # every later decode call
+    copy_gbs = None
+    if a.copy_mib > 0:
+        nbytes = a.copy_mib << 20
+        src, dst = api.DeviceBuffer(nbytes), api.DeviceBuffer(nbytes)
+        src.fill(1)
+        api.lib().openfish_amd_copy(dst.ptr, src.ptr, nbytes)
+        tc = time.perf_counter()
+        for _ in range(5):
+            api.lib().openfish_amd_copy(dst.ptr, src.ptr, nbytes)
+        copy_gbs = 5 * 2 * nbytes / 1e9 / (time.perf_counter() - tc)
+        src.free()
+        dst.free()
+    if copy_gbs:
+        stages["device_copy_GBps"] = round(copy_gbs, 1)
+        stages["scan_plus_posterior"]["frac_of_device_copy"] = round(scan_gbs / copy_gbs, 4)
 
     opt_kw = dict(beam_cut=100.0, blank_score=2.0, q_shift=q_shift, q_scale=q_scale)
     cpu = cpu_baseline(s16, state_len, opt_kw, min(a.cpu_sample, N)) if a.cpu_sample > 0 else None
