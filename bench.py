@@ -174,12 +174,12 @@ def main():
         dst.free()
 
     for _ in range(a.warmup):
-        api.openfish_decode_gpu(T, N, C, scores, state_len, opt, gpubuf)
+        api.openfish_decode_gpu_discard(T, N, C, scores, state_len, opt, gpubuf)
     api.lib().openfish_amd_sync()
     per_stage = {k: [] for k in api.STAGES}
     t0 = time.perf_counter()
     for _ in range(a.steps):
-        api.openfish_decode_gpu(T, N, C, scores, state_len, opt, gpubuf)
+        api.openfish_decode_gpu_discard(T, N, C, scores, state_len, opt, gpubuf)
         for k, v in gpubuf.timings().items():
             per_stage[k].append(v)
     api.lib().openfish_amd_sync()
@@ -208,10 +208,10 @@ def main():
     if a.scan_mode == "precise" and a.alt_steps > 0:
         api.set_scan_mode(True)
         alt = {k: [] for k in api.STAGES}
-        api.openfish_decode_gpu(T, N, C, scores, state_len, opt, gpubuf)
+        api.openfish_decode_gpu_discard(T, N, C, scores, state_len, opt, gpubuf)
         t1 = time.perf_counter()
         for _ in range(a.alt_steps):
-            api.openfish_decode_gpu(T, N, C, scores, state_len, opt, gpubuf)
+            api.openfish_decode_gpu_discard(T, N, C, scores, state_len, opt, gpubuf)
             for k, v in gpubuf.timings().items():
                 alt[k].append(v)
         alt_ms = 1e3 * (time.perf_counter() - t1) / a.alt_steps
@@ -232,13 +232,13 @@ def main():
         api.openfish_amd_decode_enqueue(T, N, C, scores, state_len, opt, bufs[0])
         for k in range(1, 2 * a.overlap_steps):
             api.openfish_amd_decode_enqueue(T, N, C, scores, state_len, opt, bufs[k % 2])
-            api.openfish_amd_decode_wait(bufs[(k - 1) % 2])
-        api.openfish_amd_decode_wait(bufs[(2 * a.overlap_steps - 1) % 2])
+            api.openfish_amd_decode_wait(bufs[(k - 1) % 2], copy=False)
+        api.openfish_amd_decode_wait(bufs[(2 * a.overlap_steps - 1) % 2], copy=False)
         sec = time.perf_counter() - t2
         overlap = {"chunks_per_s": round(2 * a.overlap_steps * N / sec, 1), "gpubufs": 2,
                    "calls": 2 * a.overlap_steps,
-                   "note": "one thread, openfish_amd_decode_enqueue/_wait alternating over two gpubufs; "
-                           "not `value`"}
+                   "note": "one thread, openfish_amd_decode_enqueue/_wait alternating over two gpubufs, results "
+                           "left in the pinned buffers; not `value`"}
 
     # what a plain streaming copy kernel reaches on this device (1 GiB each way, read + write
     # counted), as a second yardstick beside the published 8 TB/s.  Measured after the timed loops:

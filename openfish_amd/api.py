@@ -205,18 +205,31 @@ def openfish_decode_gpu(T, N, Cc, scores_dev, state_len, options, gpubuf):
     return _take(mv, N, T), _take(sq, N, T), _take(qs, N, T)
 
 
+def openfish_decode_gpu_discard(T, N, Cc, scores_dev, state_len, options, gpubuf):
+    """the same C call, results freed without a copy into numpy (what a timing loop wants: the
+    call and the caller's three free()s, nothing of this wrapper)"""
+    mv, sq, qs = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    _L.openfish_decode_gpu(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), gpubuf.handle,
+                           C.byref(mv), C.byref(sq), C.byref(qs))
+    _libc.free(mv)
+    _libc.free(sq)
+    _libc.free(qs)
+
+
 def openfish_amd_decode_enqueue(T, N, Cc, scores_dev, state_len, options, gpubuf):
     """queue one decode on the gpubuf and return at once; scores_dev must stay alive until the wait"""
     _L.openfish_amd_decode_enqueue(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), gpubuf.handle)
     gpubuf._pending_shape = (N, T)
 
 
-def openfish_amd_decode_wait(gpubuf):
+def openfish_amd_decode_wait(gpubuf, copy=True):
     """(moves, sequence, qstring) of the enqueued decode as uint8 [N, T] arrays (copies of the
-    library's pinned buffer)"""
+    library's pinned buffer); copy=False only waits (timing loops)"""
     N, T = gpubuf._pending_shape
     mv, sq, qs = C.c_void_p(), C.c_void_p(), C.c_void_p()
     _L.openfish_amd_decode_wait(gpubuf.handle, C.byref(mv), C.byref(sq), C.byref(qs))
+    if not copy:
+        return None
     out = []
     for p in (mv, sq, qs):
         buf = (C.c_uint8 * (N * T)).from_address(p.value)
