@@ -193,6 +193,10 @@ void openfish_gpubuf_free(openfish_gpubuf_t *gpubuf) {
     ofa_gpubuf_t *g = (ofa_gpubuf_t *)gpubuf;
     if (!g) return;
     if (g->magic != OFA_MAGIC) die("gpubuf was not created by openfish_gpubuf_init");
+    if (g->pending) { /* an enqueued decode still reads and writes these buffers */
+        HIP_OK(hipStreamSynchronize(g->s_side));
+        HIP_OK(hipStreamSynchronize(g->s_main));
+    }
     for (int i = 0; i < EV_COUNT; ++i) HIP_OK(hipEventDestroy(g->ev[i]));
     HIP_OK(hipStreamDestroy(g->s_main));
     HIP_OK(hipStreamDestroy(g->s_side));
@@ -210,6 +214,7 @@ static ofa_gpubuf_t *checked(const openfish_gpubuf_t *gpubuf, int T, int N, int 
     if (state_len != g->state_len || (size_t)N * (size_t)(T + 1) > (size_t)g->N * (size_t)(g->T + 1) ||
         (size_t)N * (size_t)T > (size_t)g->N * (size_t)g->T)
         die("batch shape exceeds the shape the gpubuf was created for");
+    if (g->pending) die("this gpubuf holds an enqueued decode that has not been waited for");
     return g;
 }
 
@@ -219,7 +224,10 @@ static void check_scores_any(int T, int N, int C, const void *scores, int state_
     if (T < 1 || N < 1) die("T and N must be positive");
     if (T > OFK_MAX_T) die("chunks longer than 8192 time steps are not supported");
     if (C != 4 * states_of(state_len) && !(allow_blank_column && C == 5 * states_of(state_len)))
-        die("C must be 4 * 4^state_len (one score per state and dropped base)");
+        die(allow_blank_column
+                ? "C must be 4 * 4^state_len (one score per state and dropped base) or 5 * 4^state_len (a blank "
+                  "column first)"
+                : "C must be 4 * 4^state_len (one score per state and dropped base)");
     if (!scores) die("scores_TNC is NULL");
     if (!opt) die("options is NULL");
 }
@@ -322,9 +330,6 @@ static const ofk_phred_table_t *phred_for(ofa_gpubuf_t *g, const openfish_opt_t 
 /* The three result buffers are the caller's to free (the reference's contract), so they are fresh
  * allocations every call.  They are allocated and touched while the GPU works, which takes the page
  * faults off the path between the last kernel and the return. */
-/* all three results over the main stream (the stage-level entry point) */
-static void fetch_outputs(ofa_gpubuf_t *g, int T, int N, uint8_t **moves, char **sequence, char **qstring);
-
 static void alloc_outputs(int T, int N, uint8_t **moves, char **sequence, char **qstring) {
     const size_t nt = (size_t)N * (size_t)T;
     *moves = (uint8_t *)host_alloc(nt);
@@ -335,6 +340,7 @@ static void alloc_outputs(int T, int N, uint8_t **moves, char **sequence, char *
     memset(*qstring, 0, nt);
 }
 
+/* all three results over the main stream (the stage-level entry point) */
 static void fetch_outputs(ofa_gpubuf_t *g, int T, int N, uint8_t **moves, char **sequence, char **qstring) {
     const size_t nt = (size_t)N * (size_t)T;
     HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_main));
@@ -359,7 +365,6 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
                            const int state_len, const openfish_opt_t *options) {
     const float stay = options->blank_score; /* as the reference GPU path, src/decode_hip.hip:120 */
     const size_t nt = (size_t)N * (size_t)T;
-    if (g->pending) die("this gpubuf already holds a decode that has not been waited for");
 
     join_null_stream(g);
     HIP_OK(hipEventRecord(g->ev[EV_START], g->s_main));
@@ -401,6 +406,7 @@ void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC
                          const openfish_opt_t *options, const openfish_gpubuf_t *gpubuf, uint8_t **moves,
                          char **sequence, char **qstring) {
     check_scores_any(T, N, C, scores_TNC, state_len, options, 1);
+    if (!moves || !sequence || !qstring) die("decode: output pointer is NULL");
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     const size_t nt = (size_t)N * (size_t)T;
     OPENFISH_LOG_TRACE("scores tensor dim: %d, %d, %d", T, N, C);
@@ -496,6 +502,7 @@ void openfish_amd_decode_from_tensors(int T, int N, int C, const void *scores, i
                                       const openfish_gpubuf_t *gpubuf, uint8_t **moves, char **sequence,
                                       char **qstring) {
     check_scores(T, N, C, scores, state_len, options);
+    if (!moves || !sequence || !qstring) die("decode: output pointer is NULL");
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     join_null_stream(g);
     launch_ok(ofk_beam_search(scores, bwd, (ofk_beam_slot_t *)g->pub.beam_vector, (int32_t *)g->pub.states,
