@@ -110,6 +110,13 @@ __device__ __forceinline__ int wave_sum_i(int x) {
 }
 __device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
 __device__ __forceinline__ int popc64(uint64_t x) { return __builtin_popcountll(x); }
+// Any lane with a non-zero word.  The ballot of a plain comparison is the comparison's own lane
+// mask; the ballot of a combined condition would take a detour through two more vector
+// instructions, so callers fold their condition into one integer first.
+__device__ __forceinline__ bool any_nonzero(uint32_t word) {
+    asm("" : "+v"(word));  // keeps the compiler from taking the word apart into its conditions again
+    return ballot(word != 0u) != 0;
+}
 
 __device__ __forceinline__ void wave_fence() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -208,8 +215,8 @@ struct __attribute__((aligned(16))) SlotRec {
 };
 
 struct BeamShared {
-    uint32_t hash[kW];     // hashes of the current beam, contiguous for the match sweep
-    Elem elem[kW];
+    uint32_t hash[kW + 4];  // hashes of the current beam, contiguous for the match sweep; entry kW
+    Elem elem[kW + 1];      // of both arrays is a dump slot for candidates that are not kept
     SlotRec rec[4 * kW];
     float stay_score[kW];  // only used by the serial replay of merges
     double lse[OFK_LSE_DOUBLES];
@@ -431,28 +438,38 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         {
             const uint32_t want = crc2_inverse(hash, (uint32_t)state & 3u);
             // Bit k of m says whether hash k of this half equals `want`.  Each comparison is
-            // shifted in with an add-with-carry (m = 2m + equal), two instructions per hash; the
-            // four comparisons of a vector are issued before the four adds so that no add reads
-            // a comparison result sooner than three instructions after it was written.
-            uint32_t m = 0;
-            auto four = [&](const uint4 &x) {
-                uint64_t e0, e1, e2, e3, carry;
+            // shifted into an accumulator with an add-with-carry (a = 2a + equal), two
+            // instructions per hash.  Two vectors of four hashes go through one block: the eight
+            // comparisons first, then the adds alternating between the vectors' accumulators, so
+            // that no instruction waits for the one before it.
+            auto eight = [&](const uint4 &x, const uint4 &y, uint32_t &ax, uint32_t &ay) {
+                uint64_t e0, e1, e2, e3, f0, f1, f2, f3, carry;
                 asm("v_cmp_eq_u32_e64 %[e3], %[w], %[x3]\n\t"
+                    "v_cmp_eq_u32_e64 %[f3], %[w], %[y3]\n\t"
                     "v_cmp_eq_u32_e64 %[e2], %[w], %[x2]\n\t"
+                    "v_cmp_eq_u32_e64 %[f2], %[w], %[y2]\n\t"
                     "v_cmp_eq_u32_e64 %[e1], %[w], %[x1]\n\t"
+                    "v_cmp_eq_u32_e64 %[f1], %[w], %[y1]\n\t"
                     "v_cmp_eq_u32_e64 %[e0], %[w], %[x0]\n\t"
-                    "v_addc_co_u32_e64 %[m], %[c], %[m], %[m], %[e3]\n\t"
-                    "v_addc_co_u32_e64 %[m], %[c], %[m], %[m], %[e2]\n\t"
-                    "v_addc_co_u32_e64 %[m], %[c], %[m], %[m], %[e1]\n\t"
-                    "v_addc_co_u32_e64 %[m], %[c], %[m], %[m], %[e0]"
-                    : [m] "+v"(m), [e0] "=&s"(e0), [e1] "=&s"(e1), [e2] "=&s"(e2), [e3] "=&s"(e3),
+                    "v_cmp_eq_u32_e64 %[f0], %[w], %[y0]\n\t"
+                    "v_addc_co_u32_e64 %[ax], %[c], %[ax], %[ax], %[e3]\n\t"
+                    "v_addc_co_u32_e64 %[ay], %[c], %[ay], %[ay], %[f3]\n\t"
+                    "v_addc_co_u32_e64 %[ax], %[c], %[ax], %[ax], %[e2]\n\t"
+                    "v_addc_co_u32_e64 %[ay], %[c], %[ay], %[ay], %[f2]\n\t"
+                    "v_addc_co_u32_e64 %[ax], %[c], %[ax], %[ax], %[e1]\n\t"
+                    "v_addc_co_u32_e64 %[ay], %[c], %[ay], %[ay], %[f1]\n\t"
+                    "v_addc_co_u32_e64 %[ax], %[c], %[ax], %[ax], %[e0]\n\t"
+                    "v_addc_co_u32_e64 %[ay], %[c], %[ay], %[ay], %[f0]"
+                    : [ax] "+v"(ax), [ay] "+v"(ay), [e0] "=&s"(e0), [e1] "=&s"(e1), [e2] "=&s"(e2),
+                      [e3] "=&s"(e3), [f0] "=&s"(f0), [f1] "=&s"(f1), [f2] "=&s"(f2), [f3] "=&s"(f3),
                       [c] "=&s"(carry)
-                    : [w] "v"(want), [x0] "v"(x.x), [x1] "v"(x.y), [x2] "v"(x.z), [x3] "v"(x.w));
+                    : [w] "v"(want), [x0] "v"(x.x), [x1] "v"(x.y), [x2] "v"(x.z), [x3] "v"(x.w),
+                      [y0] "v"(y.x), [y1] "v"(y.y), [y2] "v"(y.z), [y3] "v"(y.w));
             };
-            four(hq3);
-            four(hq2);
-            four(hq1);
-            four(hq0);
+            uint32_t m0 = 0, m1 = 0, m2 = 0, m3 = 0;  // four bits each, hashes 4k .. 4k+3
+            eight(hq0, hq1, m0, m1);
+            eight(hq2, hq3, m2, m3);
+            uint32_t m = (m0 | (m1 << 4)) | ((m2 | (m3 << 4)) << 8);
             m <<= 16 * h;
             {
                 // both halves of the wave looked at 16 hashes each: lanes i and i+32 join their masks
@@ -467,7 +484,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // The stay's lane fetches the step's score from the lane that holds it, folds the two,
         // keeps its half of the outcome and leaves the step's half in the step's mailbox.
         const bool mine = h == 0 && match != 0;
-        if (ballot(mine) != 0) {
+        if (any_nonzero(h == 0 ? match : 0u)) {
             const uint32_t now = (uint32_t)(t + 1);
             const uint32_t mytag = (now << 5) | (uint32_t)i;
             const int j = __builtin_ctz(match | 0x80000000u) & 31;
@@ -490,8 +507,9 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             // keep the three reads together in one LDS round trip (the compiler would otherwise
             // sink the mailbox reads below the branch that follows)
             asm volatile("" : "+v"(claimed), "+v"(box0.x), "+v"(box0.y), "+v"(box1.x), "+v"(box1.y));
-            const bool odd = mine && ((match & (match - 1)) != 0 || claimed != mytag);
-            if (ballot(odd) != 0 || (flags & 1)) {
+            // odd: a stay with several equal hashes, or a step claimed by two stays
+            const uint32_t odd = mine ? ((match & (match - 1)) | (claimed ^ mytag)) : 0u;
+            if (any_nonzero(odd) || (flags & 1)) {
                 // A stay with several equal hashes, or a step claimed by two stays (only
                 // possible after a CRC collision): replay the merges one by one in the
                 // CPU path's order, from the scores as they were before any merge.
@@ -579,18 +597,17 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const int rank1 = rank0 + (keep0 ? 1 : 0);
             const int ranks = popc64(k0) + popc64(k1) + popc64(ks & below);
             const uint32_t from = (uint32_t)i << 16;
-            if (keep0 && rank0 < kW) {
-                sh.hash[rank0] = h0;
-                sh.elem[rank0] = Elem{h0, c0, (uint32_t)(lo4 + b0) | from, c0 - g01.x};
-            }
-            if (keep1 && rank1 < kW) {
-                sh.hash[rank1] = h1;
-                sh.elem[rank1] = Elem{h1, c1, (uint32_t)(lo4 + b0 + 1) | from, c1 - g01.y};
-            }
-            if (keeps && ranks < kW) {
-                sh.hash[ranks] = hash;
-                sh.elem[ranks] = Elem{hash, cs, (uint32_t)state | from | (1u << 21), cs - gst};
-            }
+            // every lane stores all three of its candidates, the ones that are dropped into the
+            // dump slot: no branches and no exec masking on the path from the cut-off to the next beam
+            const int slot0 = (keep0 && rank0 < kW) ? rank0 : kW;
+            const int slot1 = (keep1 && rank1 < kW) ? rank1 : kW;
+            const int slots = (keeps && ranks < kW) ? ranks : kW;
+            sh.hash[slot0] = h0;
+            sh.elem[slot0] = Elem{h0, c0, (uint32_t)(lo4 + b0) | from, c0 - g01.x};
+            sh.hash[slot1] = h1;
+            sh.elem[slot1] = Elem{h1, c1, (uint32_t)(lo4 + b0 + 1) | from, c1 - g01.y};
+            sh.hash[slots] = hash;
+            sh.elem[slots] = Elem{hash, cs, (uint32_t)state | from | (1u << 21), cs - gst};
             wave_fence();
         }
         w = kept;
