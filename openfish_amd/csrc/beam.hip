@@ -217,7 +217,7 @@ struct __attribute__((aligned(16))) SlotRec {
 struct BeamShared {
     uint32_t hash[kW + 4];  // hashes of the current beam, contiguous for the match sweep; entry kW
     Elem elem[kW + 1];      // of both arrays is a dump slot for candidates that are not kept
-    SlotRec rec[4 * kW];
+    SlotRec rec[4 * kW + 1];  // entry 4 * kW is a dump slot for lanes without a merge
     float stay_score[kW];  // only used by the serial replay of merges
     double lse[OFK_LSE_DOUBLES];
     int ready;             // rows stored by the loader wave
@@ -398,8 +398,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     float gst;
     uint4 hq0, hq1, hq2, hq3;
     auto fetch_row = [&](int tt) {
-        while (rows_ready <= tt) {
-            rows_ready = observe(&sh.ready);
+        while (rows_ready <= tt) {  // the counter is one LDS word: the same value in every lane
+            rows_ready = __builtin_amdgcn_readfirstlane(observe(&sh.ready));
             if (rows_ready <= tt) __builtin_amdgcn_s_sleep(1);
         }
         const int slot = tt % LR;
@@ -494,14 +494,14 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const float o1 = __int_as_float(__builtin_amdgcn_ds_bpermute(holder, __float_as_int(c1)));
             const float other = (bi & 1) ? o1 : o0;
             const bool stay_wins = cs > other;
-            float folded = cs;
-            if (mine) folded = log_sum_exp(cs, other, sh.lse);
-            const int target = 4 * j + bi;
-            if (mine)
-                *reinterpret_cast<uint2 *>(&sh.rec[target]) =
-                    make_uint2(mytag, __float_as_uint(stay_wins ? -FLT_MAX : folded));
+            // every lane goes through the fold and the mailbox, lanes without a merge with whatever
+            // their registers hold and the dump slot as target: no exec masking on the way
+            const float folded = log_sum_exp(cs, other, sh.lse);
+            const int target = mine ? 4 * j + bi : 4 * kW;
+            *reinterpret_cast<uint2 *>(&sh.rec[target]) =
+                make_uint2(mytag, __float_as_uint(stay_wins ? -FLT_MAX : folded));
             wave_fence();
-            uint32_t claimed = mine ? sh.rec[target].tag : mytag;
+            uint32_t claimed = sh.rec[target].tag;
             uint2 box0 = *reinterpret_cast<const uint2 *>(&my_rec[0]);
             uint2 box1 = *reinterpret_cast<const uint2 *>(&my_rec[1]);
             // keep the three reads together in one LDS round trip (the compiler would otherwise
@@ -611,16 +611,15 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             wave_fence();
         }
         w = kept;
-        float rest = -FLT_MAX;
-        if (i < w) {
+        // every lane reads its slot; slots past the new width hold leftovers and are masked here
+        float rest;
+        {
             const Elem e = sh.elem[i];
+            const bool in = i < w;
             hash = e.hash;
-            score = e.score;
-            info = e.info;
-            rest = e.rest;
-        } else {
-            score = -FLT_MAX;
-            info = 0;
+            score = in ? e.score : -FLT_MAX;
+            info = in ? e.info : 0u;
+            rest = in ? e.rest : -FLT_MAX;
         }
         state = (int)(info & 0xFFFFu);
         if (t + 1 < T) fetch_row(t + 1);
@@ -644,11 +643,10 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // drop the guide term again and persist the slot (src/beam_search.c:417-427); the
         // difference was taken by the lane that held the candidate, which had the term at hand
         score = rest;
-        if (i < w) {
-            if (h == 0)
-                bv[(size_t)(t + 1) * kW + i] =
-                    (ofk_beam_slot_t)((uint32_t)state | (((info >> 16) & 31u) << 10) | (((info >> 21) & 1u) << 15));
-        }
+        // both halves hold the same element and store the same slot; slots past the width are never
+        // followed by the traceback
+        bv[(size_t)(t + 1) * kW + i] =
+            (ofk_beam_slot_t)((uint32_t)state | (((info >> 16) & 31u) << 10) | (((info >> 21) & 1u) << 15));
     }
 
     // ---- traceback from slot 0 of the last block (src/beam_search.c:432-439) ----
