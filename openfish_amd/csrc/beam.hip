@@ -147,7 +147,7 @@ __device__ __forceinline__ float log_sum_exp(float x, float y, const double *tab
     int cell = (int)(gap * 4.0f);
     cell = cell < OFK_LSE_CELLS - 1 ? cell : OFK_LSE_CELLS - 1;
     const double *c = table + cell * OFK_LSE_COEFS;
-    const double s = ((double)gap - (0.25 * cell + 0.125)) * 8.0;
+    const double s = __builtin_fma((double)gap, 8.0, -(double)(2 * cell + 1));  // (gap - centre of the cell) * 8, exactly
     double p = c[8];
 #pragma unroll
     for (int k = 7; k >= 0; --k) p = __builtin_fma(p, s, c[k]);
@@ -430,7 +430,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         float cs = (score + stay) + gst;
         publish(&sh.consumed, t + 1);  // everything this step needs of row t is in registers
         const uint32_t h0 = crc2(hash, (uint32_t)b0);
-        const uint32_t h1 = crc2(hash, (uint32_t)b0 + 1u);
+        const uint32_t h1 = h0 ^ kTab1;  // crc2(hash, b0 + 1): b0 is even, so only bit 0 of the table index flips
         SlotRec *my_rec = &sh.rec[4 * i + b0];
 
         // which previous element j has hash_j == crc^-1(hash_i, last base of i)
@@ -599,9 +599,9 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const uint32_t from = (uint32_t)i << 16;
             // every lane stores all three of its candidates, the ones that are dropped into the
             // dump slot: no branches and no exec masking on the path from the cut-off to the next beam
-            const int slot0 = (keep0 && rank0 < kW) ? rank0 : kW;
-            const int slot1 = (keep1 && rank1 < kW) ? rank1 : kW;
-            const int slots = (keeps && ranks < kW) ? ranks : kW;
+            const int slot0 = min(keep0 ? rank0 : kW, kW);
+            const int slot1 = min(keep1 ? rank1 : kW, kW);
+            const int slots = min(keeps ? ranks : kW, kW);
             sh.hash[slot0] = h0;
             sh.elem[slot0] = Elem{h0, c0, (uint32_t)(lo4 + b0) | from, c0 - g01.x};
             sh.hash[slot1] = h1;
