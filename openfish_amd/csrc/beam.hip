@@ -548,39 +548,39 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         }
 
         // cut-off (src/beam_search.c:320-381)
-        // dead lanes carry -FLT_MAX as their score, so their candidates are about -FLT_MAX too
+        // Dead lanes carry -FLT_MAX as their score, which absorbs whatever is added: their candidates
+        // are -FLT_MAX exactly, and so is the stay of the upper half from here on.
+        cs = h == 0 ? cs : -FLT_MAX;
         float best;
-        {
-            const float cs_or_none = h == 0 ? cs : -FLT_MAX;
-            asm("v_max3_f32 %0, %1, %2, %3" : "=v"(best) : "v"(c0), "v"(c1), "v"(cs_or_none));
-        }
+        asm("v_max3_f32 %0, %1, %2, %3" : "=v"(best) : "v"(c0), "v"(c1), "v"(cs));
         best = wave_max(best);
 
-        float cut = best - log_cut;
+        float cut = best - log_cut;  // may be -FLT_MAX (no cut at all): mask the dead lanes
         uint64_t k0 = ballot(c0 >= cut) & vm, k1 = ballot(c1 >= cut) & vm, ks = ballot(cs >= cut) & vs;
         int kept = popc64(k0) + popc64(k1) + popc64(ks);
         if (kept > kW) {
+            // Bisection between the cut and the best score.  Every cut tried in here lies above
+            // (-FLT_MAX + best) / 2, so dead lanes and dropped candidates never pass and the
+            // ballots need no mask.  (lo + hi) / 2 is the CPU path's (cut + hi) / 2 or
+            // (cut + lo) / 2: one of the two bounds is the cut just tried.
             float lo = cut, hi = best;
             int guesses = 1;
-            while ((kept > kW || kept < (kW * 8) / 10) && guesses < 10) {
-                if (kept > kW) {
-                    lo = cut;
-                    cut = (cut + hi) / 2.0f;
-                } else {
-                    hi = cut;
-                    cut = (cut + lo) / 2.0f;
-                }
-                k0 = ballot(c0 >= cut) & vm;
-                k1 = ballot(c1 >= cut) & vm;
-                ks = ballot(cs >= cut) & vs;
+            do {
+                const bool up = kept > kW;
+                lo = up ? cut : lo;
+                hi = up ? hi : cut;
+                cut = (lo + hi) / 2.0f;
+                k0 = ballot(c0 >= cut);
+                k1 = ballot(c1 >= cut);
+                ks = ballot(cs >= cut);
                 kept = popc64(k0) + popc64(k1) + popc64(ks);
                 ++guesses;
-            }
+            } while ((unsigned)(kept - (kW * 8) / 10) > (unsigned)(kW - (kW * 8) / 10) && guesses < 10);
             if (guesses == 10) {
                 cut = hi;
-                k0 = ballot(c0 >= cut) & vm;
-                k1 = ballot(c1 >= cut) & vm;
-                ks = ballot(cs >= cut) & vs;
+                k0 = ballot(c0 >= cut);
+                k1 = ballot(c1 >= cut);
+                ks = ballot(cs >= cut);
                 kept = popc64(k0) + popc64(k1) + popc64(ks);
             }
             if (kept > kW) kept = kW;
