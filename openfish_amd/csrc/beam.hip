@@ -565,7 +565,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             // (cut + lo) / 2: one of the two bounds is the cut just tried.
             float lo = cut, hi = best;
             int guesses = 1;
-            do {
+            for (;;) {
                 const bool up = kept > kW;
                 lo = up ? cut : lo;
                 hi = up ? hi : cut;
@@ -575,7 +575,10 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 ks = ballot(cs >= cut);
                 kept = popc64(k0) + popc64(k1) + popc64(ks);
                 ++guesses;
-            } while ((unsigned)(kept - (kW * 8) / 10) > (unsigned)(kW - (kW * 8) / 10) && guesses < 10);
+                if ((unsigned)(kept - (kW * 8) / 10) <= (unsigned)(kW - (kW * 8) / 10)) break;  // 25..32 kept
+                asm volatile("");  // two scalar branches, not one condition put together from lane masks
+                if (guesses >= 10) break;
+            }
             if (guesses == 10) {
                 cut = hi;
                 k0 = ballot(c0 >= cut);
