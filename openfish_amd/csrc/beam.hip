@@ -7,9 +7,10 @@
 // rows consumed), so the search never waits on a dependent HBM gather.  A workgroup holds
 // two or four chunks, so that its waves spread over the four SIMDs of a compute unit.
 //
-// Search wave lane layout: lane = i + 32*h holds beam element i (mirrored in both
-// halves) and the step candidates with new base 2h and 2h+1; lanes < 32 also hold
-// the stay candidate.  Candidate order is the CPU path's: steps 4i+b, then stays.
+// Search wave lane layout: lanes 2i and 2i+1 both hold beam element i; lane 2i+h holds
+// its step candidates with new base 2h and 2h+1, the even lane also its stay candidate,
+// so that lane order is the CPU path's candidate order (steps 4i+b, then stays) and
+// ranks are masked bit counts.
 // The search reproduces the CPU path (reference src/beam_search.c:117-439) to the
 // bit: same fp32 operation order, double-precision log-sum-exp for merges, the
 // same cut-off bisection, first-come compaction and final best-to-slot-0 swap.
@@ -324,9 +325,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     }
 
     // ---- search wave ----
-    const int i = lane & 31;
-    const int h = lane >> 5;
-    const uint64_t below = (((uint64_t)1 << i) - 1) * 0x100000001ull;  // elements < i, both halves
+    const int i = lane >> 1;  // lanes 2i and 2i+1 hold element i; candidate order is lane order
+    const int h = lane & 1;
 
     // seeding: the 32 best states of bwd[0] in ascending state order (src/beam_search.c:151-175)
     {
@@ -382,7 +382,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     int state = (int)(info & 0xFFFFu);
     int w = kW;
     ofk_beam_slot_t *bv = beam + (size_t)n * (size_t)(T + 1) * kW;
-    if (lane < kW) bv[lane] = (ofk_beam_slot_t)state;
+    bv[i] = (ofk_beam_slot_t)state;
 
     // The search is a chain of dependent short instructions; when it shares a SIMD with
     // throughput-bound waves (the forward scan runs at the same time) it should win the
@@ -421,7 +421,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     for (int t = 0; t < T; ++t) {
         const bool valid = i < w;
         const uint64_t vm = ballot(valid);          // live elements, both halves
-        const uint64_t vs = vm & 0xFFFFFFFFull;     // their stay candidates sit on lanes < 32
+        const uint64_t vs = vm & 0x5555555555555555ull;  // their stay candidates sit on the even lanes
         const int lo4 = (state << 2) & (S - 1);
         const float r0 = (float)r0h;
         const float r1 = (float)r1h;
@@ -472,9 +472,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             uint32_t m = (m0 | (m1 << 4)) | ((m2 | (m3 << 4)) << 8);
             m <<= 16 * h;
             {
-                // both halves of the wave looked at 16 hashes each: lanes i and i+32 join their masks
-                const auto both = __builtin_amdgcn_permlane32_swap(m, m, false, false);
-                m = both[0] | both[1];
+                // the two lanes of an element looked at 16 hashes each and join their masks
+                m |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1 /* quad_perm:[1,0,3,2] */, 0xF, 0xF, true);
             }
             const uint32_t live = w >= 32 ? 0xFFFFFFFFu : ((1u << w) - 1u);
             match = valid ? (m & live) : 0u;
@@ -489,7 +488,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const uint32_t mytag = (now << 5) | (uint32_t)i;
             const int j = __builtin_ctz(match | 0x80000000u) & 31;
             const int bi = state & 3;
-            const int holder = (j + ((bi & 2) << 4)) << 2;  // lane j + 32 * (bi >> 1), as a byte index
+            const int holder = (2 * j + (bi >> 1)) << 2;  // the lane with element j and base bi, as a byte index
             const float o0 = __int_as_float(__builtin_amdgcn_ds_bpermute(holder, __float_as_int(c0)));
             const float o1 = __int_as_float(__builtin_amdgcn_ds_bpermute(holder, __float_as_int(c1)));
             const float other = (bi & 1) ? o1 : o0;
@@ -591,14 +590,16 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
 
         // survivors in candidate order: steps (i, b) by i then b, then stays by i
         {
-            const int before = popc64(k0 & below) + popc64(k1 & below);
-            const uint32_t k0lo = (uint32_t)k0, k1lo = (uint32_t)k1;
-            const int same = h == 0 ? 0 : (int)((k0lo >> i) & 1u) + (int)((k1lo >> i) & 1u);
+            // kept candidates on lower lanes: masked bit counts
+            auto lower = [&](uint64_t mask, int start) {
+                return (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                                      __builtin_amdgcn_mbcnt_lo((uint32_t)mask, (uint32_t)start));
+            };
             const bool keep0 = valid && c0 >= cut, keep1 = valid && c1 >= cut;  // this lane's bits of k0, k1
             const bool keeps = valid && h == 0 && cs >= cut;                      // and of ks
-            const int rank0 = before + same;
+            const int rank0 = lower(k1, lower(k0, 0));
             const int rank1 = rank0 + (keep0 ? 1 : 0);
-            const int ranks = popc64(k0) + popc64(k1) + popc64(ks & below);
+            const int ranks = lower(ks, popc64(k0) + popc64(k1));
             const uint32_t from = (uint32_t)i << 16;
             // every lane stores all three of its candidates, the ones that are dropped into the
             // dump slot: no branches and no exec masking on the path from the cut-off to the next beam
@@ -632,11 +633,12 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const bool in = i < w;
             const float top_score = wave_max(in ? score : -FLT_MAX);
             const uint64_t at = ballot(in && h == 0 && score == top_score);
-            const int arg = (top_score > -FLT_MAX && at != 0) ? __builtin_ctzll(at) : 0;
+            const int arg_lane = (top_score > -FLT_MAX && at != 0) ? __builtin_ctzll(at) : 0;  // an even lane
+            const int arg = arg_lane >> 1;
             if (arg != 0) {
-                const uint32_t hash0 = lane_u(hash, 0), hasha = lane_u(hash, arg);
-                const uint32_t in0 = lane_u(info, 0), ina = lane_u(info, arg);
-                const float re0 = lane_f(rest, 0), rea = lane_f(rest, arg);
+                const uint32_t hash0 = lane_u(hash, 0), hasha = lane_u(hash, arg_lane);
+                const uint32_t in0 = lane_u(info, 0), ina = lane_u(info, arg_lane);
+                const float re0 = lane_f(rest, 0), rea = lane_f(rest, arg_lane);
                 if (i == 0) { hash = hasha; info = ina; rest = rea; }
                 if (i == arg) { hash = hash0; info = in0; rest = re0; }
                 state = (int)(info & 0xFFFFu);
