@@ -1,12 +1,11 @@
 // Double-precision exp and log for the scans, written for the narrow domains the
 // scans need so that they cost a few dozen full-rate fp64 FMAs instead of a
 // general libm call:
-//   exp_nonpos(d)   : e^d for a float d <= 0, relative error below 2^-50
-//   log_1to5(s)     : ln(s) for a float s in [1, 5] (a sum of five terms <= 1, one of
-//                     which is exactly 1), relative error below 2^-51
-//   log_1to5_tab(s) : the same from a 32-entry table of (1/c, ln c), absolute error
-//                     below 2^-51; half the instructions
-//   log1p_exp_neg   : ln(1 + e^-gap), the pairwise log-sum-exp correction
+//   exp_nonpos_ldexp(d) : e^d for a float d <= 0, absolute error below 2^-51
+//                         (relative error below 2^-50 for d >= -5.5)
+//   log_1to5_tab(s)     : ln(s) for a float s in [1, 5] (a sum of five terms <= 1, one of
+//                         which is exactly 1) from a 32-entry table of (1/c, ln c),
+//                         absolute error below 2^-51
 // The CPU path evaluates exp and log in double and then rounds to fp32 (reference
 // src/decode_cpu.c:45-49); these stand in for its libm calls.  With the errors above
 // a result can round to a different fp32 value only when the exact value lies
@@ -66,37 +65,19 @@ OFA_HD double exp_reduced(double r) {
     return __builtin_fma(p, r, 1.0);
 }
 
-// e^d, d <= 0.  Arguments below -80 are treated as -80: e^-80 = 1.8e-35 is far below
-// half an ulp of the sum it is added to (the sum contains a term equal to 1), and as a
-// first term it rounds to an fp32 value that the later 1 absorbs just the same.
-OFA_HD double exp_nonpos(float d) {
-    const double x = (double)(d > -80.0f ? d : -80.0f);
-    const double kShift = 6755399441055744.0;  // 1.5 * 2^52: adding it rounds to an integer
-    const double kLog2e = 1.4426950408889634074;
-    const double kLn2Hi = 6.93147180369123816490e-01;  // 32 significant bits: n * kLn2Hi is exact
-    const double kLn2Lo = 1.90821492927058770002e-10;
-    const double t = __builtin_fma(x, kLog2e, kShift);
-    const double n = t - kShift;
-    double r = __builtin_fma(n, -kLn2Hi, x);
-    r = __builtin_fma(n, -kLn2Lo, r);  // |r| <= ln2/2
-    const double p = exp_reduced(r);
-    // p in [0.70, 1.42]; n >= -116: scaling by 2^n is an add to the exponent field
-    const uint64_t scaled = bits_of(p) + ((uint64_t)(int64_t)(int32_t)(uint32_t)bits_of(t) << 52);
-    return double_of(scaled);
-}
-
-// The same without the clamp: the scaling is a true ldexp, which underflows to zero by
-// itself.  Needs |d| < 1e9 (the integer part of d*log2(e) is read from 32 bits).
+// e^d for a float d <= 0 (|d| < 1e9: the integer part of d*log2(e) is read from 32 bits).
+// One-step argument reduction r = d - n ln2 with ln2 rounded to double: its error, |n| 2^-54
+// relative to e^d, is |n| 2^(-54-|n|/0.69..) relative to 1, and the sums these exponentials
+// enter are at least 1 (one term of every sum is e^0).  The scaling by 2^n is a true ldexp,
+// which underflows to zero by itself.
 OFA_HD double exp_nonpos_ldexp(float d) {
     const double x = (double)d;
-    const double kShift = 6755399441055744.0;
+    const double kShift = 6755399441055744.0;  // 1.5 * 2^52: adding it rounds to an integer
     const double kLog2e = 1.4426950408889634074;
-    const double kLn2Hi = 6.93147180369123816490e-01;
-    const double kLn2Lo = 1.90821492927058770002e-10;
+    const double kLn2 = 0.69314718055994530942;
     const double t = __builtin_fma(x, kLog2e, kShift);
     const double n = t - kShift;
-    double r = __builtin_fma(n, -kLn2Hi, x);
-    r = __builtin_fma(n, -kLn2Lo, r);
+    const double r = __builtin_fma(n, -kLn2, x);  // |r| <= ln2/2 (+ 1e-14)
     const double p = exp_reduced(r);
     return __builtin_ldexp(p, (int)(uint32_t)bits_of(t));
 }
@@ -128,16 +109,6 @@ OFA_HD double log_core(double f, int k) {
     const double lu = __builtin_fma(z2 * w, p, z2);
     const double kLn2 = 0.69314718055994530942;
     return __builtin_fma((double)k, kLn2, lu);
-}
-
-// ln(s) for a float s in [1, 5]: s = 2^k * u with u in [sqrt(1/2), sqrt(2))
-OFA_HD double log_1to5(float s) {
-    const uint32_t b = bits_of(s);
-    const uint32_t frac = b & 0x007fffffu;
-    const uint32_t up = frac > 0x003504f3u ? 1u : 0u;  // mantissa above sqrt(2): use u/2, k+1
-    const int k = (int)(b >> 23) - 127 + (int)up;
-    const float u = float_of(frac | ((127u - up) << 23));
-    return log_core((double)u - 1.0, k);  // the difference is exact
 }
 
 // Table-driven ln(s), s a float in [1, 5].  The mantissa interval [1, 2) is cut into 32
@@ -173,27 +144,8 @@ OFA_HD double log_1to5_tab(float s, const LogCell *table) {
     return __builtin_fma((double)k, kLn2, lu);
 }
 
-// ln(1 + e^-gap) for a float gap in [0, 17): the correction term of log(e^x + e^y)
-// (reference src/beam_search.c:43-47), absolute error below 2^-46
-OFA_HD double log1p_exp_neg(float gap) {
-    const double x = 1.0 + exp_nonpos(-gap);  // in (1, 2]
-    const bool up = x > 1.4142135623730951;
-    const double u = up ? 0.5 * x : x;
-    return log_core(u - 1.0, up ? 1 : 0);  // the difference is exact
-}
-
-// max + ln(sum_i e^(v_i - max)) with the CPU path's roundings: fp32 differences, the
-// running sum rounded to fp32 after every term, one rounding of the final sum.
-OFA_HD float lse5_cpu_rounding(float v0, float v1, float v2, float v3, float v4, float m) {
-    float s = (float)exp_nonpos(v0 - m);
-    s = (float)((double)s + exp_nonpos(v1 - m));
-    s = (float)((double)s + exp_nonpos(v2 - m));
-    s = (float)((double)s + exp_nonpos(v3 - m));
-    s = (float)((double)s + exp_nonpos(v4 - m));
-    return (float)((double)m + log_1to5(s));
-}
-
-// the same update with the table-driven logarithm and the ldexp-scaled exponential
+// max + ln(sum_i e^(v_i - max)) with the CPU path's roundings (reference src/decode_cpu.c:45-49):
+// fp32 differences, the running sum rounded to fp32 after every term, one rounding of the final sum.
 OFA_HD float lse5_cpu_rounding_tab(float v0, float v1, float v2, float v3, float v4, float m,
                                    const LogCell *table) {
     float s = (float)exp_nonpos_ldexp(v0 - m);
