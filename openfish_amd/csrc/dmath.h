@@ -125,18 +125,22 @@ OFA_HD LogCell log_cell(int i) {
     c.lnc = -log_core(low ? 2.0 * c.inv - 1.0 : c.inv - 1.0, low ? -1 : 0);  // differences exact
     return c;
 }
-OFA_HD double log_1to5_tab(float s, const LogCell *table) {
+// Coefficients -1/8, 1/7, ..., 1/3 of the series; the caller passes them from memory the scalar
+// unit can read (on the device: constant memory), which keeps them in scalar registers for the
+// whole kernel; written as literals they would be copied into vector registers at every use.
+#define OFA_LOG_SERIES {-1.0 / 8.0, 1.0 / 7.0, -1.0 / 6.0, 1.0 / 5.0, -1.0 / 4.0, 1.0 / 3.0}
+OFA_HD double log_1to5_tab(float s, const LogCell *table, const double *series) {
     const uint32_t b = bits_of(s);
     const int k = (int)(b >> 23) - 127;
     const LogCell c = table[(b >> 18) & 31u];
     const double u = (double)float_of((b & 0x007fffffu) | 0x3f800000u);
     const double r = __builtin_fma(u, c.inv, -1.0);
-    double q = -1.0 / 8.0;
-    q = __builtin_fma(q, r, 1.0 / 7.0);
-    q = __builtin_fma(q, r, -1.0 / 6.0);
-    q = __builtin_fma(q, r, 1.0 / 5.0);
-    q = __builtin_fma(q, r, -1.0 / 4.0);
-    q = __builtin_fma(q, r, 1.0 / 3.0);
+    double q = series[0];
+    q = __builtin_fma(q, r, series[1]);
+    q = __builtin_fma(q, r, series[2]);
+    q = __builtin_fma(q, r, series[3]);
+    q = __builtin_fma(q, r, series[4]);
+    q = __builtin_fma(q, r, series[5]);
     q = __builtin_fma(q, r, -0.5);
     q = __builtin_fma(q, r, 1.0);
     const double lu = __builtin_fma(q, r, c.lnc);
@@ -147,13 +151,13 @@ OFA_HD double log_1to5_tab(float s, const LogCell *table) {
 // max + ln(sum_i e^(v_i - max)) with the CPU path's roundings (reference src/decode_cpu.c:45-49):
 // fp32 differences, the running sum rounded to fp32 after every term, one rounding of the final sum.
 OFA_HD float lse5_cpu_rounding_tab(float v0, float v1, float v2, float v3, float v4, float m,
-                                   const LogCell *table) {
+                                   const LogCell *table, const double *series) {
     float s = (float)exp_nonpos_ldexp(v0 - m);
     s = (float)((double)s + exp_nonpos_ldexp(v1 - m));
     s = (float)((double)s + exp_nonpos_ldexp(v2 - m));
     s = (float)((double)s + exp_nonpos_ldexp(v3 - m));
     s = (float)((double)s + exp_nonpos_ldexp(v4 - m));
-    return (float)((double)m + log_1to5_tab(s, table));
+    return (float)((double)m + log_1to5_tab(s, table, series));
 }
 
 }  // namespace ofa

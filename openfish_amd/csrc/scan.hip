@@ -80,12 +80,23 @@ __device__ __forceinline__ float group_max(float x) {
     return x;
 }
 
+// What the CPU-faithful logarithm reads: its table in LDS and its series coefficients.  The
+// coefficients travel as a kernel argument, which puts them into scalar registers for the whole
+// kernel (as literals the compiler copies them into vector registers at every use).
+struct LogSeries {
+    double c[6];
+};
+struct LogArgs {
+    const ofa::LogCell *cells;
+    const double *series;
+};
+
 // max + log(sum_i exp(v_i - max)), sum taken in the order v0..v4
 template <bool PRECISE>
-__device__ __forceinline__ float lse5(float v0, float v1, float v2, float v3, float v4, const ofa::LogCell *logtab) {
+__device__ __forceinline__ float lse5(float v0, float v1, float v2, float v3, float v4, const LogArgs &logtab) {
     const float m = fmaxf(fmaxf(fmaxf(v0, v1), v2), fmaxf(v3, v4));
     if constexpr (PRECISE) {
-        return ofa::lse5_cpu_rounding_tab(v0, v1, v2, v3, v4, m, logtab);
+        return ofa::lse5_cpu_rounding_tab(v0, v1, v2, v3, v4, m, logtab.cells, logtab.series);
     } else {
         float s = __builtin_amdgcn_exp2f((v0 - m) * kLog2e);
         s += __builtin_amdgcn_exp2f((v1 - m) * kLog2e);
@@ -215,7 +226,7 @@ struct FloatRun {
 
 template <int I, int SPL, bool PRECISE>
 __device__ __forceinline__ void bwd_update(float (&a)[SPL], const float4 &nx, const BwdRow<SPL> &row, float stay,
-                                           const ofa::LogCell *logtab) {
+                                           const LogArgs &logtab) {
     if constexpr (I < SPL) {
         a[I] = lse5<PRECISE>(a[I] + stay, nx.x + row.template get<0, I>(), nx.y + row.template get<1, I>(),
                              nx.z + row.template get<2, I>(), nx.w + row.template get<3, I>(), logtab);
@@ -225,7 +236,7 @@ __device__ __forceinline__ void bwd_update(float (&a)[SPL], const float4 &nx, co
 
 template <int I, int SPL, bool PRECISE>
 __device__ __forceinline__ void fwd_update(float (&f)[SPL], float p0, float p1, float p2, float p3,
-                                           const FwdRow<SPL> &row, float stay, const ofa::LogCell *logtab) {
+                                           const FwdRow<SPL> &row, float stay, const LogArgs &logtab) {
     if constexpr (I < SPL) {
         f[I] = lse5<PRECISE>(f[I] + stay, p0 + row.template get<I, 0>(), p1 + row.template get<I, 1>(),
                              p2 + row.template get<I, 2>(), p3 + row.template get<I, 3>(), logtab);
@@ -238,16 +249,17 @@ __device__ __forceinline__ void fwd_update(float (&f)[SPL], float p0, float p1, 
 // ---------------------------------------------------------------------------
 template <int S, int SPL, int DEPTH, bool PRECISE>
 __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
-    const _Float16 *__restrict__ scores, float *__restrict__ bwd, int T, int N, float stay) {
+    const _Float16 *__restrict__ scores, float *__restrict__ bwd, int T, int N, float stay, LogSeries series) {
     using Sh = Shape<S, SPL>;
     constexpr int L = Sh::kLanes;
     constexpr int Q = Sh::kQuarter;
     constexpr int H = 4 / SPL;  // lanes sharing one quad
     __shared__ __attribute__((aligned(16))) float vec[Sh::kChunks][2][S];
-    __shared__ __attribute__((aligned(16))) ofa::LogCell logtab[32];
+    __shared__ __attribute__((aligned(16))) ofa::LogCell logcells[32];
+    const LogArgs logtab{logcells, series.c};
 
     const int tid = threadIdx.x;
-    if (PRECISE && tid < 32) logtab[tid] = ofa::log_cell(tid);
+    if (PRECISE && tid < 32) logcells[tid] = ofa::log_cell(tid);
     const int g = tid / L, l = tid % L;
     const int r = l / H, c0 = (l % H) * SPL;  // own states: r + (c0 + i) * Q
     int n = blockIdx.x * Sh::kChunks + g;
@@ -306,16 +318,17 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
 template <int S, int SPL, int DEPTH, bool PRECISE>
 __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
     const _Float16 *__restrict__ scores, const float *__restrict__ bwd, float *__restrict__ post, int T,
-    int N, float stay) {
+    int N, float stay, LogSeries series) {
     using Sh = Shape<S, SPL>;
     constexpr int L = Sh::kLanes;
     constexpr int Q = Sh::kQuarter;
     __shared__ __attribute__((aligned(16))) float vec[Sh::kChunks][2][S];
     __shared__ float part[2][Sh::kChunks][Sh::kChunkWaves];
-    __shared__ __attribute__((aligned(16))) ofa::LogCell logtab[32];
+    __shared__ __attribute__((aligned(16))) ofa::LogCell logcells[32];
+    const LogArgs logtab{logcells, series.c};
 
     const int tid = threadIdx.x;
-    if (PRECISE && tid < 32) logtab[tid] = ofa::log_cell(tid);
+    if (PRECISE && tid < 32) logcells[tid] = ofa::log_cell(tid);
     const int g = tid / L, l = tid % L;
     const int s0 = SPL * l, q = s0 >> 2;  // own states s0 .. s0+SPL-1, all in quad q
     const int wave = l / 64;  // wave within the chunk
@@ -419,16 +432,18 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
 int g_scan_fast = 0;
 int g_scan_spl = 0;  // 0 = choose from the batch size
 
+const LogSeries kSeries = {OFA_LOG_SERIES};
+
 template <int S, int SPL, int DEPTH>
 int launch_bwd(const void *scores, float *bwd, int T, int N, float stay, hipStream_t st) {
     using Sh = Shape<S, SPL>;
     const int blocks = (N + Sh::kChunks - 1) / Sh::kChunks;
     if (g_scan_fast)
         hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, false>), dim3(blocks), dim3(Sh::kThreads), 0, st,
-                           static_cast<const _Float16 *>(scores), bwd, T, N, stay);
+                           static_cast<const _Float16 *>(scores), bwd, T, N, stay, kSeries);
     else
         hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, true>), dim3(blocks), dim3(Sh::kThreads), 0, st,
-                           static_cast<const _Float16 *>(scores), bwd, T, N, stay);
+                           static_cast<const _Float16 *>(scores), bwd, T, N, stay, kSeries);
     return (int)hipGetLastError();
 }
 
@@ -438,10 +453,10 @@ int launch_fwd(const void *scores, const float *bwd, float *post, int T, int N, 
     const int blocks = (N + Sh::kChunks - 1) / Sh::kChunks;
     if (g_scan_fast)
         hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, false>), dim3(blocks), dim3(Sh::kThreads), 0, st,
-                           static_cast<const _Float16 *>(scores), bwd, post, T, N, stay);
+                           static_cast<const _Float16 *>(scores), bwd, post, T, N, stay, kSeries);
     else
         hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, true>), dim3(blocks), dim3(Sh::kThreads), 0, st,
-                           static_cast<const _Float16 *>(scores), bwd, post, T, N, stay);
+                           static_cast<const _Float16 *>(scores), bwd, post, T, N, stay, kSeries);
     return (int)hipGetLastError();
 }
 

@@ -3,6 +3,8 @@
 
 #include "dmath.h"
 
+static const double kSeries[6] = OFA_LOG_SERIES;
+
 extern "C" {
 
 // largest error of exp_nonpos_ldexp against expl over the given floats: relative to the exact
@@ -25,7 +27,7 @@ double max_abs_err_log_tab(const float *s, long n) {
     for (int i = 0; i < 32; ++i) table[i] = ofa::log_cell(i);
     double worst = 0;
     for (long i = 0; i < n; ++i) {
-        const double err = (double)fabsl((long double)ofa::log_1to5_tab(s[i], table) - logl((long double)s[i]));
+        const double err = (double)fabsl((long double)ofa::log_1to5_tab(s[i], table, kSeries) - logl((long double)s[i]));
         if (err > worst) worst = err;
     }
     return worst;
@@ -47,7 +49,7 @@ long lse5_mismatches(const float *v, long n) {
         const float *p = v + 5 * i;
         float m = p[0];
         for (int k = 1; k < 5; ++k) m = m > p[k] ? m : p[k];
-        const float a = ofa::lse5_cpu_rounding_tab(p[0], p[1], p[2], p[3], p[4], m, table);
+        const float a = ofa::lse5_cpu_rounding_tab(p[0], p[1], p[2], p[3], p[4], m, table, kSeries);
         const float b = lse5_libm(p, m);
         if (memcmp(&a, &b, 4) != 0) ++bad;
     }
