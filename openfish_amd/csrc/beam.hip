@@ -195,9 +195,10 @@ struct RowRegs {
 template <int S>
 struct BeamCfg {
     static constexpr int kBits = S == 64 ? 6 : S == 256 ? 8 : 10;
-    static constexpr int kLdsRows = S >= 1024 ? 3 : 6;  // LDS ring depth
+    static constexpr int kLdsRows = S >= 1024 ? 3 : 4;  // LDS ring depth
     static constexpr int kRegRows = S >= 1024 ? 3 : 6;  // rows in flight in registers (3 or 6)
-    static constexpr int kTraceBlock = 128;             // time steps staged per traceback block
+    // time steps staged per traceback block; the staging buffers reuse the memory of the ring
+    static constexpr int kTraceBlock = S >= 256 ? 128 : 32;
 };
 
 // one beam element as handed from one time step to the next
@@ -220,21 +221,34 @@ struct BeamShared {
     Elem elem[kW + 1];      // of both arrays is a dump slot for candidates that are not kept
     SlotRec rec[4 * kW + 1];  // entry 4 * kW is a dump slot for lanes without a merge
     float stay_score[kW];  // only used by the serial replay of merges
-    double lse[OFK_LSE_DOUBLES];
     int ready;             // rows stored by the loader wave
     int consumed;          // rows the search wave is done with
 };
 
 // LDS of one chunk
 template <int S>
-struct __attribute__((aligned(16))) BeamLds {
+struct BeamRing {
     _Float16 row_s[BeamCfg<S>::kLdsRows][4 * S];
     float row_b[BeamCfg<S>::kLdsRows][S];
-    BeamShared sh;
-    ofk_beam_slot_t trace[BeamCfg<S>::kTraceBlock][kW];
-    int32_t trace_state[BeamCfg<S>::kTraceBlock];
-    uint8_t trace_move[BeamCfg<S>::kTraceBlock];
 };
+template <int S>
+struct BeamTrace {
+    ofk_beam_slot_t slot[BeamCfg<S>::kTraceBlock][kW];
+    int32_t state[BeamCfg<S>::kTraceBlock];
+    uint8_t move[BeamCfg<S>::kTraceBlock];
+};
+template <int S>
+struct __attribute__((aligned(16))) BeamLds {
+    // the ring is dead once the last time step has read its row; the traceback stages its blocks there
+    union {
+        BeamRing<S> ring;
+        BeamTrace<S> trace;
+    };
+    BeamShared sh;
+};
+static_assert(sizeof(BeamTrace<64>) <= sizeof(BeamRing<64>) && sizeof(BeamTrace<256>) <= sizeof(BeamRing<256>) &&
+                  sizeof(BeamTrace<1024>) <= sizeof(BeamRing<1024>),
+              "traceback staging must fit into the ring");
 
 // CPG chunks per workgroup.  The waves of a group are dealt round over the four SIMDs of
 // its compute unit (wave k and wave k + 4 share one), while two-wave groups were measured
@@ -256,18 +270,19 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
 
     constexpr int kGroupChunks = CPG;
     __shared__ BeamLds<S> lds[kGroupChunks];
+    __shared__ double lse[OFK_LSE_DOUBLES];  // coefficient table of the folds, one copy per workgroup
 
     // waves 0 .. kGroupChunks-1 search, the others load; wave k and wave k + kGroupChunks share a chunk
     const int wave = (int)(threadIdx.x >> 6);
     const int member = wave % kGroupChunks;
     const int n = blockIdx.x * kGroupChunks + member;
     const int lane = threadIdx.x & 63;
-    auto &row_s = lds[member].row_s;
-    auto &row_b = lds[member].row_b;
+    auto &row_s = lds[member].ring.row_s;
+    auto &row_b = lds[member].ring.row_b;
     BeamShared &sh = lds[member].sh;
-    auto &trace = lds[member].trace;
-    auto &trace_state = lds[member].trace_state;
-    auto &trace_move = lds[member].trace_move;
+    auto &trace = lds[member].trace.slot;
+    auto &trace_state = lds[member].trace.state;
+    auto &trace_move = lds[member].trace.move;
     const size_t row_stride = (size_t)N * 4 * S;
     const _Float16 *sc_n = scores + (size_t)n * 4 * S;
     const float *bw_n = bwd + (size_t)n * (size_t)(T + 1) * S;
@@ -276,6 +291,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         sh.ready = 0;
         sh.consumed = 0;
     }
+    for (int x = (int)threadIdx.x; x < OFK_LSE_DOUBLES; x += 128 * CPG) lse[x] = lse_table[x];
     __syncthreads();
     if (n >= N) return;  // odd batch: the last group has one chunk
 
@@ -353,7 +369,6 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         }
         sh.rec[lane].tag = 0;  // tags of real time steps start at 1 << 5
         sh.rec[lane + 64].tag = 0;
-        for (int x = lane; x < OFK_LSE_DOUBLES; x += 64) sh.lse[x] = lse_table[x];
         wave_fence();
         int taken = 0;
 #pragma unroll
@@ -495,7 +510,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const bool stay_wins = cs > other;
             // every lane goes through the fold and the mailbox, lanes without a merge with whatever
             // their registers hold and the dump slot as target: no exec masking on the way
-            const float folded = log_sum_exp(cs, other, sh.lse);
+            const float folded = log_sum_exp(cs, other, lse);
             const int target = mine ? 4 * j + bi : 4 * kW;
             *reinterpret_cast<uint2 *>(&sh.rec[target]) =
                 make_uint2(mytag, __float_as_uint(stay_wins ? -FLT_MAX : folded));
@@ -523,7 +538,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                         for (int b = 0; b < w; ++b) {
                             if (crc2(sh.hash[b], base) != ha) continue;
                             SlotRec *st = &sh.rec[4 * b + (int)base];
-                            const float both = log_sum_exp(sh.stay_score[a], st->step, sh.lse);
+                            const float both = log_sum_exp(sh.stay_score[a], st->step, lse);
                             if (sh.stay_score[a] > st->step) {
                                 sh.stay_score[a] = both;
                                 st->step = -FLT_MAX;
