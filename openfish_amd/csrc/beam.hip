@@ -195,10 +195,10 @@ struct RowRegs {
 template <int S>
 struct BeamCfg {
     static constexpr int kBits = S == 64 ? 6 : S == 256 ? 8 : 10;
-    static constexpr int kLdsRows = S >= 1024 ? 3 : 4;  // LDS ring depth
+    static constexpr int kLdsRows = S >= 1024 ? 3 : S >= 256 ? 4 : 6;  // LDS ring depth
     static constexpr int kRegRows = S >= 1024 ? 3 : 6;  // rows in flight in registers (3 or 6)
     // time steps staged per traceback block; the staging buffers reuse the memory of the ring
-    static constexpr int kTraceBlock = S >= 256 ? 128 : 32;
+    static constexpr int kTraceBlock = S >= 256 ? 128 : 64;
 };
 
 // one beam element as handed from one time step to the next
