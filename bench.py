@@ -267,7 +267,8 @@ def main():
         "metric": "CRF chunks decoded/sec at %s (%d states, T=%d, N=%d); achieved HBM GB/s" % (a.workload, S, T, N),
         "value": round(N / (ms_per_step / 1e3), 1), "unit": "chunks/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        # state values and scores are fp32 (fp16 inputs); the default scans evaluate exp/log in fp64
+        "vs_baseline": None, "dtype": "f32+f64" if a.scan_mode == "precise" else "f32", "data": "synthetic",
         "config": {"workload": "%s: state_len %d, S=%d, C=%d fp16 TNC, T=%d, N=%d, beam 32, beam_cut 100, blank 2.0"
                                % (a.workload, state_len, S, C, T, N),
                    "scan_mode": a.scan_mode, "seed": a.seed},
