@@ -155,6 +155,55 @@ def test_stages_against_oracle(api, state_len, T, N, stress):
     assert np.array_equal(qs, ref["qstring"])
 
 
+@pytest.mark.parametrize("seed", [101, 102, 103])
+def test_random_shapes_and_options_beam_stage_bit_exact(api, seed):
+    """random model size, shape, per-chunk score scale (flat to peaked), beam cut (none to very
+    tight), stay score and quality options: the stages after the scans, fed the CPU path's
+    tensors, reproduce the CPU path's bytes"""
+    rng = np.random.default_rng(seed)
+    for _ in range(25):
+        sl = int(rng.choice([3, 3, 4, 4, 5]))
+        T = int(rng.integers(1, 260)) if sl < 5 else int(rng.integers(1, 90))
+        N = int(rng.integers(1, 9))
+        scale = rng.choice([0.05, 0.3, 1.0, 2.5, 8.0], size=N).astype(np.float32)
+        s16 = synth.crf_scores(T, N, sl, seed=int(rng.integers(1 << 30)), chunk_scale=scale)
+        kw = dict(beam_cut=float(rng.choice([0.0, 0.5, 3.0, 17.0, 100.0, 1e6])),
+                  blank_score=float(rng.choice([2.0, 0.0, -1.5, 5.0])),
+                  q_scale=float(rng.choice([1.0, 0.95, 1.3])), q_shift=float(rng.choice([0.0, -0.2, 4.0])))
+        ref = O.decode(s16.astype(np.float32), sl, kw, nthreads=4)
+        (mv, sq, qs), _ = gpu_from_tensors(api, s16, sl, kw, ref["bwd"], ref["post"])
+        what = (sl, T, N, scale.tolist(), kw)
+        assert np.array_equal(mv, ref["moves"]), what
+        assert np.array_equal(sq, ref["sequence"]), what
+        assert np.array_equal(qs, ref["qstring"]), what
+
+
+@pytest.mark.parametrize("seed", [201, 202])
+def test_random_shapes_whole_decode(api, seed):
+    """the same kind of random cases through openfish_decode_gpu (four- and five-column input):
+    bwd identical, posterior within tolerance, moves and sequence identical"""
+    rng = np.random.default_rng(seed)
+    for _ in range(20):
+        sl = int(rng.choice([3, 4, 4, 5]))
+        T = int(rng.integers(1, 400)) if sl < 5 else int(rng.integers(1, 120))
+        N = int(rng.integers(1, 11))
+        S = 4 ** sl
+        scale = rng.choice([0.05, 0.3, 1.0, 2.5, 6.0], size=N).astype(np.float32)
+        five = bool(rng.integers(2))
+        out = synth.crf_scores(T, N, sl, seed=int(rng.integers(1 << 30)), chunk_scale=scale, five_columns=five)
+        four, dev_in = (out[0], out[1]) if five else (out, out)
+        kw = dict(beam_cut=float(rng.choice([3.0, 100.0, 1e6])), q_scale=0.95, q_shift=-0.2)
+        ref = O.decode(four.astype(np.float32), sl, kw, nthreads=4)
+        gb = api.GpuBuf(T, N, sl)
+        sc = api.upload_scores_to_hip(dev_in)
+        mv, sq, _ = api.openfish_decode_gpu(T, N, (5 if five else 4) * S, sc, sl, api.DECODER_INIT(**kw), gb)
+        what = (sl, T, N, five, scale.tolist(), kw)
+        assert np.array_equal(gb.tensor("bwd_NTC"), ref["bwd"]), what
+        close(gb.tensor("post_NTC"), ref["post"], POST_ATOL)
+        assert np.array_equal(mv, ref["moves"]), what
+        assert np.array_equal(sq, ref["sequence"]), what
+
+
 def test_fast_scan_mode_stays_within_two_ulp_of_bwd(api):
     s16 = synth.crf_scores(400, 6, 4, seed=77)
     ref = O.scans(s16.astype(np.float32), 4)
