@@ -58,7 +58,11 @@ __device__ __forceinline__ float group_sum(float x) {
     x += dpp<0x122>(x);  // row_ror:2
     x += dpp<0x121>(x);  // row_ror:1
     if constexpr (LANES >= 64) {
-        x = (lane_value(x, 0) + lane_value(x, 16)) + (lane_value(x, 32) + lane_value(x, 48));
+        // row sums travel across the rows: lane 15 of a row into the next row (rows 1 and 3), then
+        // lane 31 into rows 2 and 3; lane 63 holds the total
+        x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x142 /* row_bcast:15 */, 0xA, 0xF, false));
+        x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x143 /* row_bcast:31 */, 0xC, 0xF, false));
+        x = lane_value(x, 63);
     } else if constexpr (LANES == 32) {
         const float lo = lane_value(x, 0) + lane_value(x, 16), hi = lane_value(x, 32) + lane_value(x, 48);
         x = (threadIdx.x & 32) ? hi : lo;
