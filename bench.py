@@ -129,7 +129,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="hac", choices=sorted(WORKLOADS) + ["rotary"])
     ap.add_argument("--chunks", type=int, default=0, help="override N")
-    ap.add_argument("--scan-mode", default="precise", choices=("precise", "fast"))
+    ap.add_argument("--scan-mode", default="two_tier", choices=("two_tier", "precise", "fast"))
     ap.add_argument("--cpu-sample", type=int, default=512, help="chunks timed on the CPU path (0 = skip; capped at N)")
     ap.add_argument("--seed", type=int, default=20251125)
     ap.add_argument("--alt-steps", type=int, default=3,
@@ -160,10 +160,10 @@ def main():
     scale = synth.stress_scale(N) if stress else None
     s16 = synth.crf_scores(T, N, state_len, seed=a.seed, chunk_scale=scale, threads=16)
 
-    api.set_scan_mode(a.scan_mode == "fast")
     opt = api.DECODER_INIT(q_scale=q_scale, q_shift=q_shift)
     scores = api.upload_scores_to_hip(s16)
     gpubuf = api.GpuBuf(T, N, state_len)
+    gpubuf.set_scan_mode(a.scan_mode)
 
     if a.calibrate_copy:
         nbytes = a.calibrate_copy << 20
@@ -205,8 +205,8 @@ def main():
 
     # the same batch with the hardware-exp/log scan arithmetic, for comparison (not `value`)
     other = None
-    if a.scan_mode == "precise" and a.alt_steps > 0:
-        api.set_scan_mode(True)
+    if a.scan_mode != "fast" and a.alt_steps > 0:
+        gpubuf.set_scan_mode("fast")
         alt = {k: [] for k in api.STAGES}
         api.openfish_decode_gpu_discard(T, N, C, scores, state_len, opt, gpubuf)
         t1 = time.perf_counter()
@@ -215,7 +215,7 @@ def main():
             for k, v in gpubuf.timings().items():
                 alt[k].append(v)
         alt_ms = 1e3 * (time.perf_counter() - t1) / a.alt_steps
-        api.set_scan_mode(False)
+        gpubuf.set_scan_mode(a.scan_mode)
         fb, ff = statistics.mean(alt["bwd"]), statistics.mean(alt["fwd_post"])
         other = {"chunks_per_s": round(N / (alt_ms / 1e3), 1), "ms_per_step": round(alt_ms, 4),
                  "bwd_ms": round(fb, 4), "fwd_post_ms": round(ff, 4),
@@ -227,6 +227,7 @@ def main():
     overlap = None
     if a.overlap_steps > 0:
         bufs = [gpubuf, api.GpuBuf(T, N, state_len)]
+        bufs[1].set_scan_mode(a.scan_mode)
         api.openfish_decode_gpu(T, N, C, scores, state_len, opt, bufs[1])
         t2 = time.perf_counter()
         api.openfish_amd_decode_enqueue(T, N, C, scores, state_len, opt, bufs[0])
@@ -268,7 +269,7 @@ def main():
         "value": round(N / (ms_per_step / 1e3), 1), "unit": "chunks/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         # state values and scores are fp32 (fp16 inputs); the default scans evaluate exp/log in fp64
-        "vs_baseline": None, "dtype": "f32+f64" if a.scan_mode == "precise" else "f32", "data": "synthetic",
+        "vs_baseline": None, "dtype": "f32" if a.scan_mode == "fast" else "f32+f64", "data": "synthetic",
         "config": {"workload": "%s: state_len %d, S=%d, C=%d fp16 TNC, T=%d, N=%d, beam 32, beam_cut 100, blank 2.0"
                                % (a.workload, state_len, S, C, T, N),
                    "scan_mode": a.scan_mode, "seed": a.seed},

@@ -47,12 +47,32 @@ int openfish_amd_device_count(void);
 /* ---- stages ---- */
 
 /*
+ * Arithmetic of the scan update max + log(sum of five exponentials) (reference
+ * src/decode_cpu.c:45-49,104-108: exp and log in double, the running sum and the result
+ * rounded to fp32).
+ *   OPENFISH_AMD_SCAN_TWO_TIER (default): the update is first evaluated with the hardware's
+ *     fp32 exp/log; where that result could round to another fp32 number than the CPU path's
+ *     (it lies within the error bound of a rounding boundary) the update is re-evaluated with
+ *     double exp/log and the CPU path's roundings.  Same tensors as _PRECISE.
+ *   OPENFISH_AMD_SCAN_PRECISE: double exp/log and the CPU path's roundings for every update.
+ *   OPENFISH_AMD_SCAN_FAST: hardware fp32 exp/log only; bwd within 2 ulp.  A last-bit
+ *     difference of a scan value of magnitude 4096..8192 is a 5e-4 relative difference of the
+ *     posterior built from it, so this mode is outside the 1e-3 acceptance bar on a few
+ *     posteriors per ten million.  For measurements.
+ */
+enum openfish_amd_scan_mode {
+    OPENFISH_AMD_SCAN_TWO_TIER = 0,
+    OPENFISH_AMD_SCAN_PRECISE = 1,
+    OPENFISH_AMD_SCAN_FAST = 2
+};
+
+/*
  * Backward scan (reference backward_scan src/decode_cpu.c:13-52, GPU twin
  * bwd_scan src/scan_hip.hip:9-58).  scores: device half [T][N][C], C = 4*S.
  * bwd: device fp32 [N][T+1][S], row T is zero.
  */
 void openfish_amd_bwd_scan(int T, int N, int C, const void *scores, int state_len, float stay_score,
-                           float *bwd);
+                           int scan_mode, float *bwd);
 
 /*
  * Forward scan fused with the per-time-step posterior softmax (reference
@@ -60,7 +80,15 @@ void openfish_amd_bwd_scan(int T, int N, int C, const void *scores, int state_le
  * src/scan_hip.hip:60-200).  post: device fp32 [N][T+1][S].
  */
 void openfish_amd_fwd_post_scan(int T, int N, int C, const void *scores, int state_len,
-                                float stay_score, const float *bwd, float *post);
+                                float stay_score, int scan_mode, const float *bwd, float *post);
+
+/*
+ * Both scans and the posterior in one kernel (what openfish_decode_gpu runs by default): the
+ * backward and the forward recursion of a chunk advance side by side and meet in the middle of
+ * the chunk.  Same tensors as openfish_amd_bwd_scan followed by openfish_amd_fwd_post_scan.
+ */
+void openfish_amd_scan_posterior(int T, int N, int C, const void *scores, int state_len,
+                                 float stay_score, int scan_mode, float *bwd, float *post);
 
 /*
  * Beam search and traceback (reference beam_search_cpu src/beam_search.c:117-439).
@@ -115,12 +143,13 @@ void openfish_amd_decode_wait(const openfish_gpubuf_t *gpubuf, const uint8_t **m
 /* ---- measurement ---- */
 
 enum openfish_amd_stage {
-    OPENFISH_AMD_STAGE_BWD = 0,   /* backward scan kernel */
-    OPENFISH_AMD_STAGE_FWD = 1,   /* forward + posterior kernel */
+    OPENFISH_AMD_STAGE_BWD = 0,   /* backward scan kernel (0 when both scans ran as one kernel) */
+    OPENFISH_AMD_STAGE_FWD = 1,   /* forward + posterior kernel (0 when both scans ran as one kernel) */
     OPENFISH_AMD_STAGE_BEAM = 2,  /* beam search + traceback kernel */
     OPENFISH_AMD_STAGE_SEQ = 3,   /* quality + sequence kernel */
     OPENFISH_AMD_STAGE_TOTAL = 4, /* first launch to last kernel end, device side */
-    OPENFISH_AMD_STAGE_COUNT = 5
+    OPENFISH_AMD_STAGE_SCAN = 5,  /* both scans + posterior as one kernel (0 when they ran split) */
+    OPENFISH_AMD_STAGE_COUNT = 6
 };
 
 /*
@@ -131,27 +160,26 @@ enum openfish_amd_stage {
 int openfish_amd_last_timings(const openfish_gpubuf_t *gpubuf, float *ms, int n);
 
 /*
- * Test hook.  Bit 0 makes the beam search replay every stay/step merge serially in
- * the CPU path's order, the route it otherwise takes only after a CRC collision
- * between beam hashes; outputs must be identical with and without it.
+ * Settings of one gpubuf, read whenever a decode (or a stage that takes the gpubuf) is queued
+ * on it.  Nothing here is process-wide: two host threads with a gpubuf each do not see each
+ * other's settings (the reference keeps no state beyond the log level either,
+ * src/decode_hip.hip:83-217).  Not to be changed while a decode is enqueued on the gpubuf.
+ *
+ * scan mode: one of enum openfish_amd_scan_mode, default OPENFISH_AMD_SCAN_TWO_TIER.
+ * states per lane: tuning knob of the scans, how many of the 4^state_len states one lane
+ *   carries (4, 2 or 1); 0, the default, picks the largest value that still gives every SIMD of
+ *   the device a wavefront for the batch at hand.  Results do not depend on it.
+ * debug flags: bit 0 makes the beam search replay every stay/step merge serially in the CPU
+ *   path's order, the route it otherwise takes only after a CRC collision between beam hashes;
+ *   outputs must be identical with and without it.
+ * split scans: 0 (default) runs both scans and the posterior as one kernel, then the beam
+ *   search; 1 runs the backward scan, then the forward scan + posterior on a second stream
+ *   beside the beam search.  Same results.
  */
-void openfish_amd_set_debug_flags(int flags);
-
-/*
- * Arithmetic of the two scans.  0 (default): exp/log in double with the CPU path's
- * sequence of fp32 roundings (reference src/decode_cpu.c:45-49,104-108), so that bwd
- * and the posterior reproduce the CPU tensors.  1: hardware fp32 exp/log, faster,
- * bwd within 2 ulp; a last-bit difference of a scan value of magnitude 4096..8192 is a
- * 5e-4 relative difference of the posterior built from it.  Process-wide.
- */
-void openfish_amd_set_scan_mode(int fast);
-
-/*
- * Tuning knob of the scans: how many of the 4^state_len states one lane carries (4, 2
- * or 1).  0, the default, picks the largest value that still gives every SIMD of the
- * device a wavefront for the batch at hand.  Results do not depend on it.  Process-wide.
- */
-void openfish_amd_set_scan_states_per_lane(int spl);
+void openfish_amd_gpubuf_set_scan_mode(const openfish_gpubuf_t *gpubuf, int scan_mode);
+void openfish_amd_gpubuf_set_split_scans(const openfish_gpubuf_t *gpubuf, int split);
+void openfish_amd_gpubuf_set_scan_states_per_lane(const openfish_gpubuf_t *gpubuf, int spl);
+void openfish_amd_gpubuf_set_debug_flags(const openfish_gpubuf_t *gpubuf, int flags);
 
 /*
  * The 49 miss-probability thresholds behind the phred characters for one

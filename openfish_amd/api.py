@@ -22,7 +22,10 @@ if not os.path.exists(LIB_PATH):
 
 _L = C.CDLL(LIB_PATH)
 
-STAGES = ("bwd", "fwd_post", "beam", "sequence", "total")
+STAGES = ("bwd", "fwd_post", "beam", "sequence", "total", "scan")
+# enum openfish_amd_scan_mode
+SCAN_TWO_TIER, SCAN_PRECISE, SCAN_FAST = 0, 1, 2
+SCAN_MODES = {"two_tier": SCAN_TWO_TIER, "precise": SCAN_PRECISE, "fast": SCAN_FAST}
 
 
 class openfish_opt_t(C.Structure):
@@ -73,17 +76,19 @@ _SIGS = {
     "openfish_amd_sync": (None, []),
     "openfish_amd_copy": (None, [_vp, _vp, _sz]),
     "openfish_amd_device_count": (_i, []),
-    "openfish_amd_bwd_scan": (None, [_i, _i, _i, _vp, _i, _f, _vp]),
-    "openfish_amd_fwd_post_scan": (None, [_i, _i, _i, _vp, _i, _f, _vp, _vp]),
+    "openfish_amd_bwd_scan": (None, [_i, _i, _i, _vp, _i, _f, _i, _vp]),
+    "openfish_amd_fwd_post_scan": (None, [_i, _i, _i, _vp, _i, _f, _i, _vp, _vp]),
+    "openfish_amd_scan_posterior": (None, [_i, _i, _i, _vp, _i, _f, _i, _vp, _vp]),
+    "openfish_amd_gpubuf_set_split_scans": (None, [_bufp, _i]),
     "openfish_amd_beam_search": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _bufp]),
     "openfish_amd_sequence": (None, [_i, _i, _i, _optp, _vp, _bufp]),
     "openfish_amd_decode_enqueue": (None, [_i, _i, _i, _vp, _i, _optp, _bufp]),
     "openfish_amd_decode_wait": (None, [_bufp, _pp, _pp, _pp]),
     "openfish_amd_decode_from_tensors": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _vp, _bufp, _pp, _pp, _pp]),
     "openfish_amd_last_timings": (_i, [_bufp, C.POINTER(C.c_float), _i]),
-    "openfish_amd_set_debug_flags": (None, [_i]),
-    "openfish_amd_set_scan_mode": (None, [_i]),
-    "openfish_amd_set_scan_states_per_lane": (None, [_i]),
+    "openfish_amd_gpubuf_set_debug_flags": (None, [_bufp, _i]),
+    "openfish_amd_gpubuf_set_scan_mode": (None, [_bufp, _i]),
+    "openfish_amd_gpubuf_set_scan_states_per_lane": (None, [_bufp, _i]),
     "openfish_amd_lse_table": (None, [C.POINTER(C.c_double)]),
     "openfish_amd_phred_table": (None, [_f, _f, C.POINTER(C.c_float)]),
     "openfish_amd_version": (C.c_char_p, []),
@@ -190,6 +195,19 @@ class GpuBuf:
         dt, shp = shapes[name]
         return _device_to_host(getattr(f, name), dt, shp)
 
+    def set_scan_mode(self, mode):
+        """mode: SCAN_TWO_TIER (default), SCAN_PRECISE or SCAN_FAST, or their names"""
+        _L.openfish_amd_gpubuf_set_scan_mode(self.handle, SCAN_MODES.get(mode, mode))
+
+    def set_split_scans(self, split):
+        _L.openfish_amd_gpubuf_set_split_scans(self.handle, 1 if split else 0)
+
+    def set_scan_states_per_lane(self, spl):
+        _L.openfish_amd_gpubuf_set_scan_states_per_lane(self.handle, int(spl))
+
+    def set_debug_flags(self, flags):
+        _L.openfish_amd_gpubuf_set_debug_flags(self.handle, int(flags))
+
     def timings(self):
         """device-side milliseconds of the stages of the last openfish_decode_gpu call"""
         ms = (C.c_float * len(STAGES))()
@@ -245,12 +263,21 @@ def openfish_amd_decode_from_tensors(T, N, Cc, scores_dev, state_len, options, b
     return _take(mv, N, T), _take(sq, N, T), _take(qs, N, T)
 
 
-def openfish_amd_bwd_scan(T, N, Cc, scores_dev, state_len, stay_score, bwd_dev):
-    _L.openfish_amd_bwd_scan(T, N, Cc, _ptr(scores_dev), state_len, stay_score, _ptr(bwd_dev))
+def openfish_amd_bwd_scan(T, N, Cc, scores_dev, state_len, stay_score, bwd_dev, scan_mode=SCAN_TWO_TIER):
+    _L.openfish_amd_bwd_scan(T, N, Cc, _ptr(scores_dev), state_len, stay_score, SCAN_MODES.get(scan_mode, scan_mode),
+                             _ptr(bwd_dev))
 
 
-def openfish_amd_fwd_post_scan(T, N, Cc, scores_dev, state_len, stay_score, bwd_dev, post_dev):
-    _L.openfish_amd_fwd_post_scan(T, N, Cc, _ptr(scores_dev), state_len, stay_score, _ptr(bwd_dev), _ptr(post_dev))
+def openfish_amd_fwd_post_scan(T, N, Cc, scores_dev, state_len, stay_score, bwd_dev, post_dev,
+                               scan_mode=SCAN_TWO_TIER):
+    _L.openfish_amd_fwd_post_scan(T, N, Cc, _ptr(scores_dev), state_len, stay_score,
+                                  SCAN_MODES.get(scan_mode, scan_mode), _ptr(bwd_dev), _ptr(post_dev))
+
+
+def openfish_amd_scan_posterior(T, N, Cc, scores_dev, state_len, stay_score, bwd_dev, post_dev,
+                                scan_mode=SCAN_TWO_TIER):
+    _L.openfish_amd_scan_posterior(T, N, Cc, _ptr(scores_dev), state_len, stay_score,
+                                   SCAN_MODES.get(scan_mode, scan_mode), _ptr(bwd_dev), _ptr(post_dev))
 
 
 def openfish_amd_beam_search(T, N, Cc, scores_dev, state_len, options, bwd_dev, gpubuf):
@@ -284,18 +311,6 @@ def lse_table():
     tab = (C.c_double * (68 * 9))()
     _L.openfish_amd_lse_table(tab)
     return np.array(tab[:], dtype=np.float64).reshape(68, 9)
-
-
-def set_scan_mode(fast):
-    _L.openfish_amd_set_scan_mode(1 if fast else 0)
-
-
-def set_scan_states_per_lane(spl):
-    _L.openfish_amd_set_scan_states_per_lane(int(spl))
-
-
-def set_debug_flags(flags):
-    _L.openfish_amd_set_debug_flags(int(flags))
 
 
 def _ptr(x):

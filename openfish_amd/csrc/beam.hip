@@ -719,24 +719,19 @@ int launch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int
     return (int)hipGetLastError();
 }
 
-int g_beam_flags = 0;
-
 }  // namespace
-
-extern "C" void ofk_set_beam_flags(int flags) { g_beam_flags = flags; }
-
 
 extern "C" int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                                uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
-                               const double *lse_table, void *stream) {
+                               const double *lse_table, int flags, void *stream) {
     if (!scores || !bwd || !beam || !states || !moves || !lse_table || T < 1 || N < 1) return OFK_BAD_ARGS;
     if ((reinterpret_cast<uintptr_t>(scores) | reinterpret_cast<uintptr_t>(bwd) | reinterpret_cast<uintptr_t>(beam)) & 15u)
         return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (state_len) {
-        case 3: return launch_beam<64>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, lse_table, st);
-        case 4: return launch_beam<256>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, lse_table, st);
-        case 5: return launch_beam<1024>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, g_beam_flags, lse_table, st);
+        case 3: return launch_beam<64>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
+        case 4: return launch_beam<256>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
+        case 5: return launch_beam<1024>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
         default: return OFK_BAD_ARGS;
     }
 }

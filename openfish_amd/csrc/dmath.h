@@ -16,6 +16,7 @@
 #ifndef OPENFISH_AMD_DMATH_H
 #define OPENFISH_AMD_DMATH_H
 
+#include <math.h>
 #include <stdint.h>
 #include <string.h>
 
@@ -48,39 +49,46 @@ OFA_HD float float_of(uint32_t u) {
     return x;
 }
 
-// e^r for |r| <= ln2/2: the degree-10 polynomial of least maximal relative error on that
-// interval (2^-52.07 before rounding; found with the Remez exchange in 60-digit arithmetic).
-// The constant term is exactly 1, so e^0 = 1 exactly.
-OFA_HD double exp_reduced(double r) {
-    double p = 0x1.2727a6f878ec2p-22;
-    p = __builtin_fma(p, r, 0x1.72f9854873e44p-19);
-    p = __builtin_fma(p, r, 0x1.a01b6ce553964p-16);
-    p = __builtin_fma(p, r, 0x1.a0197a4e972fcp-13);
-    p = __builtin_fma(p, r, 0x1.6c16c0c0ac0c6p-10);
-    p = __builtin_fma(p, r, 0x1.1111112d49797p-7);
-    p = __builtin_fma(p, r, 0x1.55555555933c6p-5);
-    p = __builtin_fma(p, r, 0x1.555555554bc09p-3);
-    p = __builtin_fma(p, r, 0x1.ffffffffffe17p-2);
-    p = __builtin_fma(p, r, 0x1.000000000001dp+0);
+// Coefficients of e^r for |r| <= ln2/2, highest degree first: the degree-10 polynomial of least
+// maximal relative error on that interval (2^-52.07 before rounding; found with the Remez exchange
+// in 60-digit arithmetic); the constant term, exactly 1 so that e^0 = 1 exactly, is not in the
+// list.  Then 1.5 * 2^52 (adding it rounds to an integer), log2(e) and -ln 2.
+// A kernel passes the list as an argument, which keeps it in scalar registers; written as
+// literals the compiler copies the values into vector registers at every use.
+#define OFA_EXP_COEFS                                                                                    \
+    {0x1.2727a6f878ec2p-22, 0x1.72f9854873e44p-19, 0x1.a01b6ce553964p-16, 0x1.a0197a4e972fcp-13,         \
+     0x1.6c16c0c0ac0c6p-10, 0x1.1111112d49797p-7,  0x1.55555555933c6p-5,  0x1.555555554bc09p-3,          \
+     0x1.ffffffffffe17p-2,  0x1.000000000001dp+0,  6755399441055744.0,    1.4426950408889634074,         \
+     -0.69314718055994530942}
+#define OFA_EXP_COEF_COUNT 13
+OFA_HD double exp_reduced(double r, const double *c) {
+    double p = c[0];
+    p = __builtin_fma(p, r, c[1]);
+    p = __builtin_fma(p, r, c[2]);
+    p = __builtin_fma(p, r, c[3]);
+    p = __builtin_fma(p, r, c[4]);
+    p = __builtin_fma(p, r, c[5]);
+    p = __builtin_fma(p, r, c[6]);
+    p = __builtin_fma(p, r, c[7]);
+    p = __builtin_fma(p, r, c[8]);
+    p = __builtin_fma(p, r, c[9]);
     return __builtin_fma(p, r, 1.0);
 }
 
-// e^d for a float d <= 0 (|d| < 1e9: the integer part of d*log2(e) is read from 32 bits).
-// One-step argument reduction r = d - n ln2 with ln2 rounded to double: its error, |n| 2^-54
-// relative to e^d, is |n| 2^(-54-|n|/0.69..) relative to 1, and the sums these exponentials
+// e^x for a double x (|x| < 1e9: the integer part of x*log2(e) is read from 32 bits); the scans
+// call it with x = a float d <= 0.
+// One-step argument reduction r = x - n ln2 with ln2 rounded to double: its error, |n| 2^-54
+// relative to e^x, is |n| 2^(-54-|n|/0.69..) relative to 1, and the sums these exponentials
 // enter are at least 1 (one term of every sum is e^0).  The scaling by 2^n is a true ldexp,
 // which underflows to zero by itself.
-OFA_HD double exp_nonpos_ldexp(float d) {
-    const double x = (double)d;
-    const double kShift = 6755399441055744.0;  // 1.5 * 2^52: adding it rounds to an integer
-    const double kLog2e = 1.4426950408889634074;
-    const double kLn2 = 0.69314718055994530942;
-    const double t = __builtin_fma(x, kLog2e, kShift);
-    const double n = t - kShift;
-    const double r = __builtin_fma(n, -kLn2, x);  // |r| <= ln2/2 (+ 1e-14)
-    const double p = exp_reduced(r);
+OFA_HD double exp_ldexp(double x, const double *c) {
+    const double t = __builtin_fma(x, c[11], c[10]);
+    const double n = t - c[10];
+    const double r = __builtin_fma(n, c[12], x);  // |r| <= ln2/2 (+ 1e-14)
+    const double p = exp_reduced(r, c);
     return __builtin_ldexp(p, (int)(uint32_t)bits_of(t));
 }
+OFA_HD double exp_nonpos_ldexp(float d, const double *c) { return exp_ldexp((double)d, c); }
 
 // k*ln2 + ln(1 + f) for f in [sqrt(1/2) - 1, sqrt(2) - 1]:
 // ln(1 + f) = 2 atanh(z), z = f / (2 + f), |z| <= 0.1716.
@@ -148,16 +156,100 @@ OFA_HD double log_1to5_tab(float s, const LogCell *table, const double *series) 
     return __builtin_fma((double)k, kLn2, lu);
 }
 
+// RN32(m + ln s) as the CPU path forms it: the sum in double, one rounding.  ln 1 is exactly 0 on
+// the CPU path; the table logarithm returns about 1e-18 there, which would show in a result whose
+// m is zero.
+OFA_HD float add_log_rounded(float m, float s, const LogCell *table, const double *series) {
+    const float r = (float)((double)m + log_1to5_tab(s, table, series));
+    return s == 1.0f ? m : r;
+}
+
 // max + ln(sum_i e^(v_i - max)) with the CPU path's roundings (reference src/decode_cpu.c:45-49):
 // fp32 differences, the running sum rounded to fp32 after every term, one rounding of the final sum.
 OFA_HD float lse5_cpu_rounding_tab(float v0, float v1, float v2, float v3, float v4, float m,
-                                   const LogCell *table, const double *series) {
-    float s = (float)exp_nonpos_ldexp(v0 - m);
-    s = (float)((double)s + exp_nonpos_ldexp(v1 - m));
-    s = (float)((double)s + exp_nonpos_ldexp(v2 - m));
-    s = (float)((double)s + exp_nonpos_ldexp(v3 - m));
-    s = (float)((double)s + exp_nonpos_ldexp(v4 - m));
-    return (float)((double)m + log_1to5_tab(s, table, series));
+                                   const LogCell *table, const double *series, const double *ec) {
+    float s = (float)exp_nonpos_ldexp(v0 - m, ec);
+    s = (float)((double)s + exp_nonpos_ldexp(v1 - m, ec));
+    s = (float)((double)s + exp_nonpos_ldexp(v2 - m, ec));
+    s = (float)((double)s + exp_nonpos_ldexp(v3 - m, ec));
+    s = (float)((double)s + exp_nonpos_ldexp(v4 - m, ec));
+    return add_log_rounded(m, s, table, series);
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Two-tier evaluation.  lse5_estimate computes the same quantity with the fp32 hardware
+// exponential and logarithm and decides whether its rounded result is certain to be the fp32
+// number the CPU path (reference src/decode_cpu.c:45-49) produces.  Where it is not certain
+// ("unsettled"), the caller evaluates lse5_cpu_rounding_tab instead.
+//
+// With d_i = v_i - m (fp32, as on the CPU path) the CPU path's result is RN32(m + ln s_cpu),
+// s_cpu the fp32 running sum of the double exponentials.  The estimate forms
+//   t_i = RN32(d_i * c),  E_i = exp2(t_i),  s~ = fp32 running sum of E_i,  l2 = log2(s~),
+//   r~ = RN32(m + l2 * ln2f)          (one fused multiply-add)
+// and x~ = m + l2 * ln2f differs from x = m + ln s_cpu by at most eps, all terms in units of
+// 2^-24 = 5.96e-8:
+//   5.00  s_cpu against the exact sum S of the e^{d_i}: five roundings of at most half an ulp
+//         of a partial sum <= s
+//   4.00  s~ against the exact sum of the E_i: four fp32 additions
+//   1.43 (S-1)/S   v_exp_f32: largest relative error found over every input in [-160, 0] is
+//         1.423 * 2^-24; the term with d = 0 is exactly 1
+//   0.88  argument of exp2: t_i = d_i c (1 + p), |p| <= 2^-24 + 1.34e-8 (c rounded to fp32), a
+//         relative error |d_i| p of E_i; sum_i |d_i| e^{d_i} / S <= 0.718
+//   0.70 * 2^k  v_log_f32: largest absolute error found over every input in [1, 5.01] is
+//         1.0, 2.0, 4.0 * 2^-24 for s~ in [1,2), [2,4), [4,5.01]; times ln 2
+//   0.12  ln2f against ln 2 (1.9e-9 * l2), rounding of the residual below, second-order terms
+// i.e. 11.41, 12.46, 13.91 for the three binades of s~; eps below adds 3 %.
+//
+// r~ is settled when no rounding boundary lies within eps of x~: with rho = x~ - r~ (exact up
+// to one rounding: r~ - m is exact by Sterbenz' lemma once |m| >= 3.3, and smaller |m| are
+// never settled because half an ulp of r~ is then below eps) and h = half an ulp of r~, the
+// distance from x~ to the nearer boundary is h - |rho|, unless r~ is a power of two, whose lower
+// boundary is only h/2 away: those (and zero) count as unsettled.
+// ---------------------------------------------------------------------------------------------
+OFA_HD float exp2_hw(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_exp2f(x);
+#else
+    return exp2f(x);
+#endif
+}
+OFA_HD float log2_hw(float x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_logf(x);
+#else
+    return log2f(x);
+#endif
+}
+
+struct Lse5Estimate {
+    float value;
+    bool settled;
+};
+OFA_HD Lse5Estimate lse5_estimate(float v0, float v1, float v2, float v3, float v4, float m) {
+    const float kLog2e = 1.44269504088896340736f, kLn2 = 0.69314718055994530942f;
+    float s = exp2_hw((v0 - m) * kLog2e);
+    s += exp2_hw((v1 - m) * kLog2e);
+    s += exp2_hw((v2 - m) * kLog2e);
+    s += exp2_hw((v3 - m) * kLog2e);
+    s += exp2_hw((v4 - m) * kLog2e);
+    const float l2 = log2_hw(s);
+    Lse5Estimate e;
+    e.value = __builtin_fmaf(l2, kLn2, m);
+    const float rho = __builtin_fmaf(l2, kLn2, -(e.value - m));
+    const uint32_t rb = bits_of(e.value);
+    const float h = float_of((rb & 0x7f800000u) - (24u << 23));  // negative or huge-negative below 2^-102
+    const float eps = __builtin_fmaf(float_of(bits_of(s) & 0x7f800000u), 0.65e-7f, 6.35e-7f);
+    e.settled = (h - __builtin_fabsf(rho) > eps) && (rb & 0x007fffffu) != 0;
+    return e;
+}
+
+// the scan update in two tiers: the estimate where it is settled, the CPU roundings elsewhere
+OFA_HD float lse5_two_tier(float v0, float v1, float v2, float v3, float v4, float m, const LogCell *table,
+                           const double *series, const double *ec) {
+    const Lse5Estimate e = lse5_estimate(v0, v1, v2, v3, v4, m);
+    if (e.settled) return e.value;
+    return lse5_cpu_rounding_tab(v0, v1, v2, v3, v4, m, table, series, ec);
 }
 
 }  // namespace ofa

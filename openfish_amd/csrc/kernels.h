@@ -21,15 +21,26 @@ extern "C" {
 /* one persisted beam slot, 16 bit: state[9:0] | prev[14:10] | stay[15] */
 typedef uint16_t ofk_beam_slot_t;
 
-/* 0 (default): scans reproduce the CPU path's double exp/log and fp32 roundings;
- * 1: scans use the hardware fp32 exp/log (faster, last-bit differences). */
-void ofk_set_scan_fast(int on);
-/* states per lane of the scans: 4, 2 or 1; 0 (default) chooses from the batch size */
-void ofk_set_scan_states_per_lane(int spl);
-int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, float stay,
-                 void *stream);
+/* Arithmetic of the scan update max + log(sum exp):
+ *   OFK_SCAN_TWO_TIER  hardware fp32 exp/log where its rounded result is provably the CPU path's,
+ *                      the CPU path's double exp/log and fp32 roundings elsewhere (same results
+ *                      as OFK_SCAN_PRECISE);
+ *   OFK_SCAN_PRECISE   the CPU path's double exp/log and fp32 roundings everywhere;
+ *   OFK_SCAN_FAST      hardware fp32 exp/log everywhere (last-bit differences).
+ * spl: states per lane, 4, 2 or 1; 0 chooses from the batch size. */
+#define OFK_SCAN_TWO_TIER 0
+#define OFK_SCAN_PRECISE 1
+#define OFK_SCAN_FAST 2
+int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, float stay, int mode,
+                 int spl, void *stream);
 int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N,
-                      int state_len, float stay, void *stream);
+                      int state_len, float stay, int mode, int spl, void *stream);
+/* Both sweeps and the posterior in one kernel: the forward and backward recursions of a chunk run
+ * side by side in one workgroup and meet in the middle of the chunk (same tensors as
+ * ofk_bwd_scan followed by ofk_fwd_post_scan).  Rows 0 .. T/2-1 of post hold forward values
+ * while the kernel runs. */
+int ofk_scan_posterior(const void *scores, float *bwd, float *post, int T, int N, int state_len,
+                       float stay, int mode, int spl, void *stream);
 /* Table behind log(1 + e^-gap), the correction of a pairwise log-sum-exp, for gap in
  * [0, 17): OFK_LSE_CELLS cells of width 1/4, each a degree-8 polynomial in
  * s = 8 * (gap - centre) in [-1, 1], coefficients lowest degree first.  Built on the
@@ -40,10 +51,9 @@ int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, 
 
 int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                     uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
-                    const double *lse_table, void *stream);
-/* bit 0: replay every stay/step merge one by one in CPU order (the path otherwise taken
+                    const double *lse_table, int flags, void *stream);
+/* flags bit 0: replay every stay/step merge one by one in CPU order (the path otherwise taken
  * only after a hash collision); results must not change.  For tests. */
-void ofk_set_beam_flags(int flags);
 /* Phred characters run from '"' (34, q = 1) to 'S' (83, q = 50).  thr[j] is the smallest
  * miss probability x whose character is at most 82 - j (2.0f if no x in [0,1] reaches it),
  * so that char(x) = 83 - #{j : x >= thr[j]}. */

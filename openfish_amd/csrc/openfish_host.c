@@ -117,6 +117,7 @@ void openfish_amd_lse_table(double *out) { build_lse_table(out); }
 #define OFA_MAGIC 0x6f66616d64677075ull /* "ofamdgpu" */
 
 enum { EV_JOIN, EV_START, EV_BWD_END, EV_BEAM_START, EV_BEAM_END, EV_FWD_END, EV_SEQ_START, EV_SEQ_END, EV_COUNT };
+/* with both sweeps in one kernel EV_BWD_END marks its end and EV_FWD_END is not recorded */
 
 typedef struct {
     openfish_gpubuf_t pub; /* first: the pointer handed to callers is this struct */
@@ -133,6 +134,11 @@ typedef struct {
     int timed;
     int pending;           /* a decode has been enqueued and not yet waited for */
     int pend_T, pend_N;    /* its shape */
+    int pend_split;        /* how its scans were queued (which events were recorded) */
+    int scan_mode;         /* OFK_SCAN_*: arithmetic of the scans of this gpubuf's decodes */
+    int scan_spl;          /* states per lane of the scans, 0 = chosen from the batch size */
+    int debug_flags;       /* bit 0: serial replay of the beam search's merges */
+    int split_scans;       /* 1: backward sweep, then forward sweep beside the beam search; 0: both sweeps in one kernel */
     ofk_phred_table_t phred; /* thresholds for (phred_shift, phred_scale) */
     float phred_shift, phred_scale;
     int phred_valid;
@@ -369,27 +375,44 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
     join_null_stream(g);
     HIP_OK(hipEventRecord(g->ev[EV_START], g->s_main));
     scores_TNC = four_columns(g, T, N, C, scores_TNC, state_len);
-    launch_ok(ofk_bwd_scan(scores_TNC, g->pub.bwd_NTC, T, N, state_len, stay, g->s_main), "bwd_scan");
-    HIP_OK(hipEventRecord(g->ev[EV_BWD_END], g->s_main));
+    g->pend_split = g->split_scans;
+    if (!g->split_scans) {
+        /* both sweeps and the posterior in one kernel, then the beam search, all on one stream */
+        launch_ok(ofk_scan_posterior(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->scan_mode,
+                                     g->scan_spl, g->s_main), "scan_posterior");
+        HIP_OK(hipEventRecord(g->ev[EV_BWD_END], g->s_main));
+        HIP_OK(hipEventRecord(g->ev[EV_BEAM_START], g->s_main));
+        launch_ok(ofk_beam_search(scores_TNC, g->pub.bwd_NTC, (ofk_beam_slot_t *)g->pub.beam_vector,
+                                  (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, log_beam_cut(options),
+                                  stay, g->lse_table, g->debug_flags, g->s_main), "beam_search");
+        HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_main));
+        /* the moves are final once the beam search is: they travel while the sequence stage runs */
+        HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BEAM_END], 0));
+        HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_side));
+    } else {
+        launch_ok(ofk_bwd_scan(scores_TNC, g->pub.bwd_NTC, T, N, state_len, stay, g->scan_mode, g->scan_spl, g->s_main),
+                  "bwd_scan");
+        HIP_OK(hipEventRecord(g->ev[EV_BWD_END], g->s_main));
 
-    /* The beam search is the longer of the two stages that follow and wants its workgroups (large
-     * LDS blocks) resident before the forward sweep fills the compute units: it stays on the stream
-     * the backward sweep ran on and so starts first; the forward sweep follows through an event. */
-    HIP_OK(hipEventRecord(g->ev[EV_BEAM_START], g->s_main));
-    launch_ok(ofk_beam_search(scores_TNC, g->pub.bwd_NTC, (ofk_beam_slot_t *)g->pub.beam_vector,
-                              (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, log_beam_cut(options),
-                              stay, g->lse_table, g->s_main), "beam_search");
-    HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_main));
+        /* The beam search is the longer of the two stages that follow and wants its workgroups (large
+         * LDS blocks) resident before the forward sweep fills the compute units: it stays on the stream
+         * the backward sweep ran on and so starts first; the forward sweep follows through an event. */
+        HIP_OK(hipEventRecord(g->ev[EV_BEAM_START], g->s_main));
+        launch_ok(ofk_beam_search(scores_TNC, g->pub.bwd_NTC, (ofk_beam_slot_t *)g->pub.beam_vector,
+                                  (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, log_beam_cut(options),
+                                  stay, g->lse_table, g->debug_flags, g->s_main), "beam_search");
+        HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_main));
 
-    HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BWD_END], 0));
-    launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->s_side),
-              "fwd_post_scan");
-    HIP_OK(hipEventRecord(g->ev[EV_FWD_END], g->s_side));
-    /* the moves are final once the beam search is: they travel while the sequence stage runs */
-    HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BEAM_END], 0));
-    HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_side));
+        HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BWD_END], 0));
+        launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->scan_mode,
+                                    g->scan_spl, g->s_side), "fwd_post_scan");
+        HIP_OK(hipEventRecord(g->ev[EV_FWD_END], g->s_side));
+        /* the moves are final once the beam search is: they travel while the sequence stage runs */
+        HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BEAM_END], 0));
+        HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_side));
+        HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_FWD_END], 0));
+    }
 
-    HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_FWD_END], 0));
     HIP_OK(hipEventRecord(g->ev[EV_SEQ_START], g->s_main));
     launch_ok(ofk_sequence(g->pub.post_NTC, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data,
                            g->pub.base_probs, g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N,
@@ -449,8 +472,14 @@ int openfish_amd_last_timings(const openfish_gpubuf_t *gpubuf, float *ms, int n)
     ofa_gpubuf_t *g = (ofa_gpubuf_t *)gpubuf;
     if (!g || g->magic != OFA_MAGIC) die("gpubuf was not created by openfish_gpubuf_init");
     if (!g->timed || !ms || n < 1) return 0;
-    HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_BWD], g->ev[EV_START], g->ev[EV_BWD_END]));
-    HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_FWD], g->ev[EV_BWD_END], g->ev[EV_FWD_END]));
+    if (g->pend_split) {
+        HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_BWD], g->ev[EV_START], g->ev[EV_BWD_END]));
+        HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_FWD], g->ev[EV_BWD_END], g->ev[EV_FWD_END]));
+        g->ms[OPENFISH_AMD_STAGE_SCAN] = 0.0f;
+    } else {
+        g->ms[OPENFISH_AMD_STAGE_BWD] = g->ms[OPENFISH_AMD_STAGE_FWD] = 0.0f;
+        HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_SCAN], g->ev[EV_START], g->ev[EV_BWD_END]));
+    }
     HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_BEAM], g->ev[EV_BEAM_START], g->ev[EV_BEAM_END]));
     HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_SEQ], g->ev[EV_SEQ_START], g->ev[EV_SEQ_END]));
     HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_TOTAL], g->ev[EV_START], g->ev[EV_SEQ_END]));
@@ -461,18 +490,35 @@ int openfish_amd_last_timings(const openfish_gpubuf_t *gpubuf, float *ms, int n)
 
 /* ---- stages ---------------------------------------------------------------- */
 
-void openfish_amd_bwd_scan(int T, int N, int C, const void *scores, int state_len, float stay_score, float *bwd) {
+static void check_scan_mode(int scan_mode) {
+    if (scan_mode != OFK_SCAN_TWO_TIER && scan_mode != OFK_SCAN_PRECISE && scan_mode != OFK_SCAN_FAST)
+        die("scan mode must be OPENFISH_AMD_SCAN_TWO_TIER, _PRECISE or _FAST");
+}
+
+void openfish_amd_bwd_scan(int T, int N, int C, const void *scores, int state_len, float stay_score, int scan_mode,
+                           float *bwd) {
     openfish_opt_t o = DECODER_INIT;
     check_scores(T, N, C, scores, state_len, &o);
-    launch_ok(ofk_bwd_scan(scores, bwd, T, N, state_len, stay_score, NULL), "bwd_scan");
+    check_scan_mode(scan_mode);
+    launch_ok(ofk_bwd_scan(scores, bwd, T, N, state_len, stay_score, scan_mode, 0, NULL), "bwd_scan");
     HIP_OK(hipStreamSynchronize(0));
 }
 
 void openfish_amd_fwd_post_scan(int T, int N, int C, const void *scores, int state_len, float stay_score,
-                                const float *bwd, float *post) {
+                                int scan_mode, const float *bwd, float *post) {
     openfish_opt_t o = DECODER_INIT;
     check_scores(T, N, C, scores, state_len, &o);
-    launch_ok(ofk_fwd_post_scan(scores, bwd, post, T, N, state_len, stay_score, NULL), "fwd_post_scan");
+    check_scan_mode(scan_mode);
+    launch_ok(ofk_fwd_post_scan(scores, bwd, post, T, N, state_len, stay_score, scan_mode, 0, NULL), "fwd_post_scan");
+    HIP_OK(hipStreamSynchronize(0));
+}
+
+void openfish_amd_scan_posterior(int T, int N, int C, const void *scores, int state_len, float stay_score,
+                                 int scan_mode, float *bwd, float *post) {
+    openfish_opt_t o = DECODER_INIT;
+    check_scores(T, N, C, scores, state_len, &o);
+    check_scan_mode(scan_mode);
+    launch_ok(ofk_scan_posterior(scores, bwd, post, T, N, state_len, stay_score, scan_mode, 0, NULL), "scan_posterior");
     HIP_OK(hipStreamSynchronize(0));
 }
 
@@ -482,7 +528,7 @@ void openfish_amd_beam_search(int T, int N, int C, const void *scores, int state
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     launch_ok(ofk_beam_search(scores, bwd, (ofk_beam_slot_t *)g->pub.beam_vector, (int32_t *)g->pub.states,
                               g->pub.moves, T, N, state_len, log_beam_cut(options), options->blank_score,
-                              g->lse_table, NULL),
+                              g->lse_table, g->debug_flags, NULL),
               "beam_search");
     HIP_OK(hipStreamSynchronize(0));
 }
@@ -507,7 +553,7 @@ void openfish_amd_decode_from_tensors(int T, int N, int C, const void *scores, i
     join_null_stream(g);
     launch_ok(ofk_beam_search(scores, bwd, (ofk_beam_slot_t *)g->pub.beam_vector, (int32_t *)g->pub.states,
                               g->pub.moves, T, N, state_len, log_beam_cut(options), options->blank_score,
-                              g->lse_table, g->s_main), "beam_search");
+                              g->lse_table, g->debug_flags, g->s_main), "beam_search");
     launch_ok(ofk_sequence(post, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data, g->pub.base_probs,
                            g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N, state_len,
                            phred_for(g, options), g->s_main), "sequence");
@@ -602,10 +648,30 @@ int openfish_amd_device_count(void) {
     return n;
 }
 
-void openfish_amd_set_debug_flags(int flags) { ofk_set_beam_flags(flags & 1); }
+/* Settings live in the gpubuf and are read when a decode is enqueued on it, so callers with one
+ * gpubuf each (one per host thread) do not see each other's settings. */
+static ofa_gpubuf_t *owned(const openfish_gpubuf_t *gpubuf) {
+    ofa_gpubuf_t *g = (ofa_gpubuf_t *)gpubuf;
+    if (!g || g->magic != OFA_MAGIC) die("gpubuf was not created by openfish_gpubuf_init");
+    return g;
+}
 
-void openfish_amd_set_scan_mode(int fast) { ofk_set_scan_fast(fast ? 1 : 0); }
+void openfish_amd_gpubuf_set_debug_flags(const openfish_gpubuf_t *gpubuf, int flags) {
+    owned(gpubuf)->debug_flags = flags & 1;
+}
 
-void openfish_amd_set_scan_states_per_lane(int spl) { ofk_set_scan_states_per_lane(spl); }
+void openfish_amd_gpubuf_set_scan_mode(const openfish_gpubuf_t *gpubuf, int scan_mode) {
+    check_scan_mode(scan_mode);
+    owned(gpubuf)->scan_mode = scan_mode;
+}
+
+void openfish_amd_gpubuf_set_split_scans(const openfish_gpubuf_t *gpubuf, int split) {
+    owned(gpubuf)->split_scans = split ? 1 : 0;
+}
+
+void openfish_amd_gpubuf_set_scan_states_per_lane(const openfish_gpubuf_t *gpubuf, int spl) {
+    if (spl != 0 && spl != 1 && spl != 2 && spl != 4) die("states per lane must be 0 (automatic), 1, 2 or 4");
+    owned(gpubuf)->scan_spl = spl;
+}
 
 const char *openfish_amd_version(void) { return "openfish-amd gfx950"; }

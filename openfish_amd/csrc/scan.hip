@@ -29,6 +29,8 @@
 // default for that reason.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "dmath.h"
 #include "kernels.h"
 
@@ -84,33 +86,6 @@ __device__ __forceinline__ float group_max(float x) {
     return x;
 }
 
-// What the CPU-faithful logarithm reads: its table in LDS and its series coefficients.  The
-// coefficients travel as a kernel argument, which puts them into scalar registers for the whole
-// kernel (as literals the compiler copies them into vector registers at every use).
-struct LogSeries {
-    double c[6];
-};
-struct LogArgs {
-    const ofa::LogCell *cells;
-    const double *series;
-};
-
-// max + log(sum_i exp(v_i - max)), sum taken in the order v0..v4
-template <bool PRECISE>
-__device__ __forceinline__ float lse5(float v0, float v1, float v2, float v3, float v4, const LogArgs &logtab) {
-    const float m = fmaxf(fmaxf(fmaxf(v0, v1), v2), fmaxf(v3, v4));
-    if constexpr (PRECISE) {
-        return ofa::lse5_cpu_rounding_tab(v0, v1, v2, v3, v4, m, logtab.cells, logtab.series);
-    } else {
-        float s = __builtin_amdgcn_exp2f((v0 - m) * kLog2e);
-        s += __builtin_amdgcn_exp2f((v1 - m) * kLog2e);
-        s += __builtin_amdgcn_exp2f((v2 - m) * kLog2e);
-        s += __builtin_amdgcn_exp2f((v3 - m) * kLog2e);
-        s += __builtin_amdgcn_exp2f((v4 - m) * kLog2e);
-        return __builtin_fmaf(__builtin_amdgcn_logf(s), kLn2, m);
-    }
-}
-
 template <bool MULTIWAVE>
 __device__ __forceinline__ void chunk_sync() {
     if constexpr (MULTIWAVE) {
@@ -129,6 +104,100 @@ __device__ __forceinline__ void chunk_sync() {
     }
 }
 
+// What the CPU-faithful logarithm reads: its table in LDS and its series coefficients.  The
+// coefficients travel as a kernel argument, which puts them into scalar registers for the whole
+// kernel (as literals the compiler copies them into vector registers at every use).
+struct LogSeries {
+    double c[6];
+    double e[OFA_EXP_COEF_COUNT];  // exponential: polynomial, rounding shift, log2(e), -ln 2
+};
+struct LogArgs {
+    const ofa::LogCell *cells;
+    const double *series;
+    const double *expc;
+    float *lanes;  // 64 floats of LDS owned by the calling wave (two-tier updates only)
+};
+
+// Two-tier update, second tier.  `value` is the estimate of a lane's update, `unsettled` says
+// that it may differ from the CPU path's result.  A wave usually has none, one or two such
+// lanes, and evaluating the CPU roundings under their execution mask would cost the whole wave
+// the five double exponentials, the running sum and the logarithm one after another.  Instead
+// the unsettled lanes hand their inputs (d_0..d_4 = v_i - m, and m) to groups of eight lanes
+// through LDS: lane 8q+j of group q computes the double exponential of d_j of the q-th unsettled
+// lane, the fp32 running sum travels from lane to lane by DPP row shifts (so lane 8q+4 ends with
+// the CPU path's sum), that lane takes the logarithm, adds m in double and rounds once, and the
+// result returns to its owner through a lane permute.  More than eight unsettled lanes take
+// further trips (only the first few dozen time steps have that many: values are small there and
+// an ulp is tiny; the kernels run those steps with the double arithmetic throughout).
+#ifdef OFK_TIER_STATS
+__device__ unsigned long long g_tier_stats[4];  // wave-level calls, calls with unsettled lanes, trips, unsettled lanes
+#endif
+
+__device__ __forceinline__ float resolve_unsettled(float value, bool unsettled, float v0, float v1, float v2, float v3,
+                                                   float v4, float m, const LogArgs &logtab) {
+    uint64_t mask = __builtin_amdgcn_ballot_w64(unsettled);
+#ifdef OFK_TIER_STATS
+    if ((threadIdx.x & 63) == 0) {
+        atomicAdd(&g_tier_stats[0], 1ull);
+        if (mask) atomicAdd(&g_tier_stats[1], 1ull);
+        atomicAdd(&g_tier_stats[2], (unsigned long long)((__builtin_popcountll(mask) + 7) / 8));
+        atomicAdd(&g_tier_stats[3], (unsigned long long)__builtin_popcountll(mask));
+    }
+#endif
+    if (mask == 0) return value;
+    __builtin_amdgcn_s_setprio(3);  // the chunk's other waves wait at the barrier for this one
+    const int lane = threadIdx.x & 63;
+    int rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+    if (!unsettled) rank = -1;
+    do {  // eight unsettled lanes per trip
+        if ((unsigned)rank < 8u) {
+            float *slot = logtab.lanes + 8 * rank;
+            *reinterpret_cast<float4 *>(slot) = make_float4(v0 - m, v1 - m, v2 - m, v3 - m);
+            *reinterpret_cast<float2 *>(slot + 4) = make_float2(v4 - m, m);
+        }
+        chunk_sync<false>();
+        const float x = logtab.lanes[lane];
+        chunk_sync<false>();  // the next trip (or call) of this wave writes the slots again
+        const double e = ofa::exp_ldexp((double)x, logtab.expc);
+        float s = (float)e;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) s = (float)((double)dpp<0x111>(s) + e);  // row_shr:1: the sum so far, from the lane below
+        const float m_of_group = dpp<0x101>(x);  // row_shl:1: lane 8q+4 reads m from lane 8q+5
+        const float r = ofa::add_log_rounded(m_of_group, s, logtab.cells, logtab.series);
+        const float mine = __int_as_float(__builtin_amdgcn_ds_bpermute((8 * (rank & 7) + 4) << 2, __float_as_int(r)));
+        if ((unsigned)rank < 8u) value = mine;
+        rank -= 8;
+        mask = __builtin_amdgcn_ballot_w64(rank >= 0);
+    } while (mask != 0);
+    __builtin_amdgcn_s_setprio(0);
+    return value;
+}
+
+// max + log(sum_i exp(v_i - max)), sum taken in the order v0..v4
+template <int MODE>
+__device__ __forceinline__ float lse5(float v0, float v1, float v2, float v3, float v4, const LogArgs &logtab) {
+    const float m = fmaxf(fmaxf(fmaxf(v0, v1), v2), fmaxf(v3, v4));
+    if constexpr (MODE == OFK_SCAN_PRECISE) {
+        return ofa::lse5_cpu_rounding_tab(v0, v1, v2, v3, v4, m, logtab.cells, logtab.series, logtab.expc);
+    } else if constexpr (MODE == OFK_SCAN_TWO_TIER) {
+        const ofa::Lse5Estimate e = ofa::lse5_estimate(v0, v1, v2, v3, v4, m);
+#if defined(OFK_EXPERIMENT_NO_RESOLVE)
+        return e.settled ? e.value : e.value + 0.0f * m;
+#elif defined(OFK_EXPERIMENT_BALLOT_ONLY)
+        return __builtin_amdgcn_ballot_w64(!e.settled) == 0x123456789ull ? m : e.value;
+#else
+        return resolve_unsettled(e.value, !e.settled, v0, v1, v2, v3, v4, m, logtab);
+#endif
+    } else {
+        float s = __builtin_amdgcn_exp2f((v0 - m) * kLog2e);
+        s += __builtin_amdgcn_exp2f((v1 - m) * kLog2e);
+        s += __builtin_amdgcn_exp2f((v2 - m) * kLog2e);
+        s += __builtin_amdgcn_exp2f((v3 - m) * kLog2e);
+        s += __builtin_amdgcn_exp2f((v4 - m) * kLog2e);
+        return __builtin_fmaf(__builtin_amdgcn_logf(s), kLn2, m);
+    }
+}
+
 template <int S, int SPL>
 struct Shape {
     static constexpr int kLanes = S / SPL;                            // lanes per chunk
@@ -143,39 +212,57 @@ struct Shape {
     static constexpr int kQuarter = S / 4;
 };
 
-// The scores one lane needs for one time step, as loaded (fp16).
+// x + (float)h for the fp16 value h in the low (HI = 0) or high half of a 32-bit register, in one
+// instruction: v_fma_mix_f32 converts the half operand on the fly, the product with 1.0 is
+// exact, so the result is the correctly rounded fp32 sum, bit for bit what v_cvt_f32_f16
+// followed by v_add_f32 gives (checked for every fp16 bit pattern, subnormals included).
+template <int HI>
+__device__ __forceinline__ float add_half(uint32_t word, float x) {
+    float r;
+    if constexpr (HI)
+        asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(word), "v"(x));
+    else
+        asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(word), "v"(x));
+    return r;
+}
+
+// The scores one lane needs for one time step, as loaded: fp16 pairs in 32-bit words.
 // Backward: transition b of own state i is element 4b + i of the lane's window.
 template <int SPL>
 struct BwdRow;
 template <>
 struct BwdRow<4> {
-    half8 v[2];
+    uint4 v[2];
     __device__ __forceinline__ void load(const _Float16 *p) {
-        v[0] = reinterpret_cast<const half8 *>(p)[0];
-        v[1] = reinterpret_cast<const half8 *>(p)[1];
+        v[0] = reinterpret_cast<const uint4 *>(p)[0];
+        v[1] = reinterpret_cast<const uint4 *>(p)[1];
     }
     template <int B, int I>
-    __device__ __forceinline__ float get() const { return (float)v[(4 * B + I) / 8][(4 * B + I) % 8]; }
+    __device__ __forceinline__ float add(float x) const {
+        constexpr int e = 4 * B + I;
+        const uint32_t w[8] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w};
+        return add_half<e % 2>(w[e / 2], x);
+    }
 };
 template <>
 struct BwdRow<2> {
-    half2v v[4];
+    uint32_t v[4];
     __device__ __forceinline__ void load(const _Float16 *p) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) v[b] = *reinterpret_cast<const half2v *>(p + 4 * b);
+        for (int b = 0; b < 4; ++b) v[b] = *reinterpret_cast<const uint32_t *>(p + 4 * b);
     }
     template <int B, int I>
-    __device__ __forceinline__ float get() const { return (float)v[B][I]; }
+    __device__ __forceinline__ float add(float x) const { return add_half<I>(v[B], x); }
 };
 template <>
 struct BwdRow<1> {
-    _Float16 v[4];
+    uint32_t v[4];  // one fp16 value each, in the low half
     __device__ __forceinline__ void load(const _Float16 *p) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) v[b] = p[4 * b];
+        for (int b = 0; b < 4; ++b) v[b] = *reinterpret_cast<const uint16_t *>(p + 4 * b);
     }
     template <int B, int I>
-    __device__ __forceinline__ float get() const { return (float)v[B]; }
+    __device__ __forceinline__ float add(float x) const { return add_half<0>(v[B], x); }
 };
 
 // Forward: transition b into own state i is element 4i + b of the lane's window.
@@ -183,27 +270,35 @@ template <int SPL>
 struct FwdRow;
 template <>
 struct FwdRow<4> {
-    half8 v[2];
+    uint4 v[2];
     __device__ __forceinline__ void load(const _Float16 *p) {
-        v[0] = reinterpret_cast<const half8 *>(p)[0];
-        v[1] = reinterpret_cast<const half8 *>(p)[1];
+        v[0] = reinterpret_cast<const uint4 *>(p)[0];
+        v[1] = reinterpret_cast<const uint4 *>(p)[1];
     }
     template <int I, int B>
-    __device__ __forceinline__ float get() const { return (float)v[(4 * I + B) / 8][(4 * I + B) % 8]; }
+    __device__ __forceinline__ float add(float x) const {
+        constexpr int e = 4 * I + B;
+        const uint32_t w[8] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w};
+        return add_half<e % 2>(w[e / 2], x);
+    }
 };
 template <>
 struct FwdRow<2> {
-    half8 v;
-    __device__ __forceinline__ void load(const _Float16 *p) { v = *reinterpret_cast<const half8 *>(p); }
+    uint4 v;
+    __device__ __forceinline__ void load(const _Float16 *p) { v = *reinterpret_cast<const uint4 *>(p); }
     template <int I, int B>
-    __device__ __forceinline__ float get() const { return (float)v[4 * I + B]; }
+    __device__ __forceinline__ float add(float x) const {
+        constexpr int e = 4 * I + B;
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        return add_half<e % 2>(w[e / 2], x);
+    }
 };
 template <>
 struct FwdRow<1> {
-    half4 v;
-    __device__ __forceinline__ void load(const _Float16 *p) { v = *reinterpret_cast<const half4 *>(p); }
+    uint2 v;
+    __device__ __forceinline__ void load(const _Float16 *p) { v = *reinterpret_cast<const uint2 *>(p); }
     template <int I, int B>
-    __device__ __forceinline__ float get() const { return (float)v[B]; }
+    __device__ __forceinline__ float add(float x) const { return add_half<B % 2>(B / 2 ? v.y : v.x, x); }
 };
 
 // SPL consecutive floats in global or shared memory
@@ -228,30 +323,30 @@ struct FloatRun {
     }
 };
 
-template <int I, int SPL, bool PRECISE>
+template <int I, int SPL, int MODE>
 __device__ __forceinline__ void bwd_update(float (&a)[SPL], const float4 &nx, const BwdRow<SPL> &row, float stay,
                                            const LogArgs &logtab) {
     if constexpr (I < SPL) {
-        a[I] = lse5<PRECISE>(a[I] + stay, nx.x + row.template get<0, I>(), nx.y + row.template get<1, I>(),
-                             nx.z + row.template get<2, I>(), nx.w + row.template get<3, I>(), logtab);
-        bwd_update<I + 1, SPL, PRECISE>(a, nx, row, stay, logtab);
+        a[I] = lse5<MODE>(a[I] + stay, row.template add<0, I>(nx.x), row.template add<1, I>(nx.y),
+                          row.template add<2, I>(nx.z), row.template add<3, I>(nx.w), logtab);
+        bwd_update<I + 1, SPL, MODE>(a, nx, row, stay, logtab);
     }
 }
 
-template <int I, int SPL, bool PRECISE>
+template <int I, int SPL, int MODE>
 __device__ __forceinline__ void fwd_update(float (&f)[SPL], float p0, float p1, float p2, float p3,
                                            const FwdRow<SPL> &row, float stay, const LogArgs &logtab) {
     if constexpr (I < SPL) {
-        f[I] = lse5<PRECISE>(f[I] + stay, p0 + row.template get<I, 0>(), p1 + row.template get<I, 1>(),
-                             p2 + row.template get<I, 2>(), p3 + row.template get<I, 3>(), logtab);
-        fwd_update<I + 1, SPL, PRECISE>(f, p0, p1, p2, p3, row, stay, logtab);
+        f[I] = lse5<MODE>(f[I] + stay, row.template add<I, 0>(p0), row.template add<I, 1>(p1),
+                          row.template add<I, 2>(p2), row.template add<I, 3>(p3), logtab);
+        fwd_update<I + 1, SPL, MODE>(f, p0, p1, p2, p3, row, stay, logtab);
     }
 }
 
 // ---------------------------------------------------------------------------
 // backward: bwd[n][t][s] for t = T..0
 // ---------------------------------------------------------------------------
-template <int S, int SPL, int DEPTH, bool PRECISE>
+template <int S, int SPL, int DEPTH, int MODE>
 __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
     const _Float16 *__restrict__ scores, float *__restrict__ bwd, int T, int N, float stay, LogSeries series) {
     using Sh = Shape<S, SPL>;
@@ -260,10 +355,11 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
     constexpr int H = 4 / SPL;  // lanes sharing one quad
     __shared__ __attribute__((aligned(16))) float vec[Sh::kChunks][2][S];
     __shared__ __attribute__((aligned(16))) ofa::LogCell logcells[32];
-    const LogArgs logtab{logcells, series.c};
-
+    __shared__ __attribute__((aligned(16))) float tier_lanes[MODE == OFK_SCAN_TWO_TIER ? Sh::kThreads : 64];
     const int tid = threadIdx.x;
-    if (PRECISE && tid < 32) logcells[tid] = ofa::log_cell(tid);
+    const LogArgs logtab{logcells, series.c, series.e, tier_lanes + (MODE == OFK_SCAN_TWO_TIER ? (tid & ~63) : 0)};
+
+    if (MODE != OFK_SCAN_FAST && tid < 32) logcells[tid] = ofa::log_cell(tid);
     const int g = tid / L, l = tid % L;
     const int r = l / H, c0 = (l % H) * SPL;  // own states: r + (c0 + i) * Q
     int n = blockIdx.x * Sh::kChunks + g;
@@ -303,7 +399,7 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
                 if (t - DEPTH >= 0) ring[k].load(sp + (size_t)(t - DEPTH) * row_stride);
                 chunk_sync<Sh::kMultiWave>();
                 const float4 nx = *reinterpret_cast<const float4 *>(&vec[g][buf][4 * r]);
-                bwd_update<0, SPL, PRECISE>(a, nx, row, stay, logtab);
+                bwd_update<0, SPL, MODE>(a, nx, row, stay, logtab);
                 buf ^= 1;
 #pragma unroll
                 for (int i = 0; i < SPL; ++i) vec[g][buf][r + (c0 + i) * Q] = a[i];
@@ -319,7 +415,7 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
 // ---------------------------------------------------------------------------
 // forward + posterior: post[n][t][s] = softmax_s(fwd[t][s] + bwd[n][t][s]), t = 0..T
 // ---------------------------------------------------------------------------
-template <int S, int SPL, int DEPTH, bool PRECISE>
+template <int S, int SPL, int DEPTH, int MODE>
 __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
     const _Float16 *__restrict__ scores, const float *__restrict__ bwd, float *__restrict__ post, int T,
     int N, float stay, LogSeries series) {
@@ -329,10 +425,11 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
     __shared__ __attribute__((aligned(16))) float vec[Sh::kChunks][2][S];
     __shared__ float part[2][Sh::kChunks][Sh::kChunkWaves];
     __shared__ __attribute__((aligned(16))) ofa::LogCell logcells[32];
-    const LogArgs logtab{logcells, series.c};
-
+    __shared__ __attribute__((aligned(16))) float tier_lanes[MODE == OFK_SCAN_TWO_TIER ? Sh::kThreads : 64];
     const int tid = threadIdx.x;
-    if (PRECISE && tid < 32) logcells[tid] = ofa::log_cell(tid);
+    const LogArgs logtab{logcells, series.c, series.e, tier_lanes + (MODE == OFK_SCAN_TWO_TIER ? (tid & ~63) : 0)};
+
+    if (MODE != OFK_SCAN_FAST && tid < 32) logcells[tid] = ofa::log_cell(tid);
     const int g = tid / L, l = tid % L;
     const int s0 = SPL * l, q = s0 >> 2;  // own states s0 .. s0+SPL-1, all in quad q
     const int wave = l / 64;  // wave within the chunk
@@ -425,7 +522,7 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
                     const float p1 = vec[g][buf][q + Q];
                     const float p2 = vec[g][buf][q + 2 * Q];
                     const float p3 = vec[g][buf][q + 3 * Q];
-                    fwd_update<0, SPL, PRECISE>(f, p0, p1, p2, p3, row, stay, logtab);
+                    fwd_update<0, SPL, MODE>(f, p0, p1, p2, p3, row, stay, logtab);
                     buf ^= 1;
                 }
             }
@@ -433,34 +530,391 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
     }
 }
 
-int g_scan_fast = 0;
-int g_scan_spl = 0;  // 0 = choose from the batch size
+// ---------------------------------------------------------------------------
+// Both sweeps in one kernel, meeting in the middle.
+//
+// The forward recursion does not depend on the backward one; only the posterior needs
+// both.  A chunk is served by two groups of lanes of one workgroup, one per direction,
+// which doubles the wavefronts in flight (the separate sweeps leave the device at one or
+// two waves per SIMD at 512 chunks of 256 states, where every wave issues at half the rate
+// the SIMD could take).
+//   phase 1: the backward lanes run t = T-1 .. H and write bwd[t]; the forward lanes run
+//            t = 0 .. H-1 and park fwd[t] in post[t];
+//   middle : the partition function max_s(fwd[H][s] + bwd[H][s]) fixes the exponent shift
+//            of the softmax (it is the same at every time step);
+//   phase 2: the forward lanes run t = H .. T reading bwd[t] (written in phase 1), the
+//            backward lanes run t = H-1 .. 0 reading the parked fwd[t]; both write the
+//            posterior, the backward lanes over the parked values.
+// HBM traffic: every score twice, bwd written once, half of it read once, post written once
+// and half of it written and read once more as fwd: (T+1) S 4 bytes above the two separate
+// sweeps.  One block barrier per time step serves both directions.
+// ---------------------------------------------------------------------------
+template <int S, int SPL>
+struct FusedShape {
+    static constexpr int kLanes = S / SPL;                 // lanes per direction and chunk
+    static constexpr int kRoleWaves = kLanes / 64;         // whole waves: a wave has one direction
+    static constexpr int kChunkThreads = 2 * kLanes;
+    static constexpr int kChunks = kChunkThreads >= 512 ? 1 : 512 / kChunkThreads;
+    static constexpr int kThreads = kChunks * kChunkThreads;
+    static constexpr int kQuarter = S / 4;
+    static_assert(kLanes % 64 == 0, "a direction owns whole wavefronts");
+};
 
-const LogSeries kSeries = {OFA_LOG_SERIES};
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
+// `count` steps, DEPTH of them unrolled per trip: step(k, j, checked) with k = j % DEPTH a
+// compile-time index; in unchecked trips j + DEPTH + SLACK < count holds for every step, i.e.
+// every prefetch DEPTH steps ahead is in range (of a tensor with SLACK rows fewer than steps).
+template <int DEPTH, int SLACK = 0, typename Step>
+__device__ __forceinline__ void pipelined(int count, Step &&step) {
+    int j0 = 0;
+    for (; j0 + 2 * DEPTH + SLACK <= count; j0 += DEPTH)
+        static_for<DEPTH>([&](auto k) { step(k, j0 + (int)k, std::false_type{}); });
+    for (; j0 < count; j0 += DEPTH)
+        static_for<DEPTH>([&](auto k) {
+            if (j0 + (int)k < count) step(k, j0 + (int)k, std::true_type{});
+        });
+}
+
+__device__ __forceinline__ void block_barrier_lds() { chunk_sync<true>(); }
+
+template <int S, int SPL, int DEPTH, int MODE>
+__global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_kernel(
+    const _Float16 *__restrict__ scores, float *__restrict__ bwd, float *__restrict__ post, int T, int N, float stay,
+    LogSeries series) {
+    using Sh = FusedShape<S, SPL>;
+    constexpr int L = Sh::kLanes;
+    constexpr int Q = Sh::kQuarter;
+    constexpr int RW = Sh::kRoleWaves;
+    constexpr int H4 = 4 / SPL;  // backward lanes sharing one quad
+    constexpr int kWarmup = 32;  // time steps of either sweep evaluated in double before the two tiers take over
+    __shared__ __attribute__((aligned(16))) float vecB[Sh::kChunks][2][S];
+    __shared__ __attribute__((aligned(16))) float vecF[Sh::kChunks][2][S];
+    __shared__ float part[Sh::kChunks][2][2][RW];  // [chunk][direction][parity][wave]
+    __shared__ float shift_of[Sh::kChunks];
+    __shared__ __attribute__((aligned(16))) ofa::LogCell logcells[32];
+    __shared__ __attribute__((aligned(16))) float tier_lanes[MODE == OFK_SCAN_TWO_TIER ? Sh::kThreads : 64];
+    const int tid = threadIdx.x;
+    const LogArgs logtab{logcells, series.c, series.e, tier_lanes + (MODE == OFK_SCAN_TWO_TIER ? (tid & ~63) : 0)};
+
+    if (MODE != OFK_SCAN_FAST && tid < 32) logcells[tid] = ofa::log_cell(tid);
+    const int g = tid / Sh::kChunkThreads, u = tid % Sh::kChunkThreads;
+    const int forward = __builtin_amdgcn_readfirstlane(u / L);
+    const int l = u % L, wave = l / 64;
+    int n = blockIdx.x * Sh::kChunks + g;
+    const bool live = Sh::kChunks == 1 || n < N;
+    if (!live) n = N - 1;
+
+    const int H = T / 2;  // forward: rows 0..H-1 in phase 1, H..T in phase 2
+    const ptrdiff_t row_stride = (ptrdiff_t)N * 4 * S;  // fp16 elements between time steps
+    const size_t chunk_off = (size_t)n * (size_t)(T + 1) * S;
+
+    if (!forward) {
+        // ------------------------------ backward lanes ------------------------------
+        const int r = l / H4, c0 = (l % H4) * SPL;  // own states: r + (c0 + i) * Q
+        const _Float16 *sp = scores + (size_t)n * 4 * S + 16 * r + c0;
+        float *out = bwd + chunk_off + r + c0 * Q;
+        float *pp = post + chunk_off + r + c0 * Q;
+        float a[SPL];
+#pragma unroll
+        for (int i = 0; i < SPL; ++i) {
+            a[i] = 0.f;
+            vecB[g][0][r + (c0 + i) * Q] = 0.f;
+            if (live) out[(size_t)T * S + i * Q] = 0.f;
+        }
+        int buf = 0;
+        BwdRow<SPL> ring[DEPTH];
+        __syncthreads();  // log table, initial vectors
+
+        // phase 1: t = T-1 .. H.  Values start at zero, where an ulp is far below the error bound of
+        // the estimate: in two-tier mode the first kWarmup steps use the double arithmetic throughout.
+        const int cnt1 = T - H;
+        auto sweep1 = [&](auto mode, int first, int count) {
+            constexpr int M = decltype(mode)::value;
+            const _Float16 *row0 = sp + (ptrdiff_t)(T - 1 - first) * row_stride;
+            float *o0 = out + (ptrdiff_t)(T - 1 - first) * S;
+            static_for<DEPTH>([&](auto k) {
+                if ((int)k < count) ring[k].load(row0 - (ptrdiff_t)k * row_stride);
+            });
+            pipelined<DEPTH>(count, [&](auto k, int j, auto checked) {
+                const BwdRow<SPL> row = ring[k];
+                if (!checked || j + DEPTH < count) ring[k].load(row0 - (ptrdiff_t)(j + DEPTH) * row_stride);
+                block_barrier_lds();
+                const float4 nx = *reinterpret_cast<const float4 *>(&vecB[g][buf][4 * r]);
+                bwd_update<0, SPL, M>(a, nx, row, stay, logtab);
+                buf ^= 1;
+#pragma unroll
+                for (int i = 0; i < SPL; ++i) vecB[g][buf][r + (c0 + i) * Q] = a[i];
+                if (live) {
+#pragma unroll
+                    for (int i = 0; i < SPL; ++i) o0[i * Q - (ptrdiff_t)j * S] = a[i];
+                }
+            });
+        };
+        const int warm = MODE == OFK_SCAN_TWO_TIER ? (cnt1 < kWarmup ? cnt1 : kWarmup) : 0;
+        if constexpr (MODE == OFK_SCAN_TWO_TIER) sweep1(std::integral_constant<int, OFK_SCAN_PRECISE>{}, 0, warm);
+        sweep1(std::integral_constant<int, MODE>{}, warm, cnt1 - warm);
+        // forward lanes may run one step fewer in phase 1: cnt1 - H is 0 or 1; they wait here
+        // middle: bwd[H..T] visible to the forward lanes, fwd[0..H-1] to these; the shift
+        __syncthreads();
+        block_barrier_lds();  // the forward lanes exchange their partial maxima
+        block_barrier_lds();  // ... and publish the shift
+        const float shift = shift_of[g];
+
+        // phase 2: t = H-1 .. 0, posterior of row t from the parked fwd[t]
+        const int cnt2 = H;
+        int pb = 0;
+        float e_prev[SPL];
+        {
+            const _Float16 *row0 = sp + (ptrdiff_t)(H - 1) * row_stride;
+            float *o0 = out + (ptrdiff_t)(H - 1) * S;
+            float *p0 = pp + (ptrdiff_t)(H - 1) * S;
+            float fring[DEPTH][SPL];
+            static_for<DEPTH>([&](auto k) {
+                if ((int)k < cnt2) {
+                    ring[k].load(row0 - (ptrdiff_t)k * row_stride);
+#pragma unroll
+                    for (int i = 0; i < SPL; ++i) fring[k][i] = p0[i * Q - (ptrdiff_t)k * S];
+                }
+            });
+            pipelined<DEPTH>(cnt2, [&](auto k, int j, auto checked) {
+                const BwdRow<SPL> row = ring[k];
+                float fv[SPL];
+#pragma unroll
+                for (int i = 0; i < SPL; ++i) fv[i] = fring[k][i];
+                if (!checked || j + DEPTH < cnt2) {
+                    ring[k].load(row0 - (ptrdiff_t)(j + DEPTH) * row_stride);
+#pragma unroll
+                    for (int i = 0; i < SPL; ++i) fring[k][i] = p0[i * Q - (ptrdiff_t)(j + DEPTH) * S];
+                }
+                block_barrier_lds();
+                if (j > 0) {  // posterior of the previous row: its total is complete now
+                    float total = part[g][0][pb ^ 1][0];
+#pragma unroll
+                    for (int w = 1; w < RW; ++w) total += part[g][0][pb ^ 1][w];
+                    const float inv = __builtin_amdgcn_rcpf(total);
+                    if (live) {
+#pragma unroll
+                        for (int i = 0; i < SPL; ++i) p0[i * Q - (ptrdiff_t)(j - 1) * S] = e_prev[i] * inv;
+                    }
+                }
+                const float4 nx = *reinterpret_cast<const float4 *>(&vecB[g][buf][4 * r]);
+                bwd_update<0, SPL, MODE>(a, nx, row, stay, logtab);
+                buf ^= 1;
+                float total = 0.f;
+#pragma unroll
+                for (int i = 0; i < SPL; ++i) {
+                    vecB[g][buf][r + (c0 + i) * Q] = a[i];
+                    e_prev[i] = __builtin_amdgcn_exp2f(((fv[i] + a[i]) - shift) * kLog2e);
+                    total += e_prev[i];
+                }
+                total = group_sum<64>(total);
+                if ((tid & 63) == 0) part[g][0][pb][wave] = total;
+                pb ^= 1;
+                if (live) {
+#pragma unroll
+                    for (int i = 0; i < SPL; ++i) o0[i * Q - (ptrdiff_t)j * S] = a[i];
+                }
+            });
+        }
+        block_barrier_lds();
+        if (cnt2 > 0) {
+            float total = part[g][0][pb ^ 1][0];
+#pragma unroll
+            for (int w = 1; w < RW; ++w) total += part[g][0][pb ^ 1][w];
+            const float inv = __builtin_amdgcn_rcpf(total);
+            if (live) {
+#pragma unroll
+                for (int i = 0; i < SPL; ++i) pp[i * Q] = e_prev[i] * inv;  // row 0
+            }
+        }
+        // the forward lanes take T - H + 1 barriers in phase 2, these took H + 1
+        for (int x = H + 1; x < T - H + 1; ++x) block_barrier_lds();
+    } else {
+        // ------------------------------ forward lanes ------------------------------
+        const int s0 = SPL * l, q = s0 >> 2;  // own states s0 .. s0+SPL-1, all in quad q
+        const _Float16 *sp = scores + (size_t)n * 4 * S + 4 * s0;
+        const float *bp = bwd + chunk_off + s0;
+        float *pp = post + chunk_off + s0;
+        float f[SPL];
+#pragma unroll
+        for (int i = 0; i < SPL; ++i) {
+            f[i] = 0.f;
+            vecF[g][0][s0 + i] = 0.f;
+        }
+        int buf = 0;
+        FwdRow<SPL> ring[DEPTH];
+        __syncthreads();
+
+        // phase 1: t = 0 .. H-1, fwd[t] parked in post[t]; warm-up as for the backward lanes
+        const int cnt1 = H;
+        auto sweep1 = [&](auto mode, int first, int count) {
+            constexpr int M = decltype(mode)::value;
+            const _Float16 *row0 = sp + (ptrdiff_t)first * row_stride;
+            float *p0p = pp + (size_t)first * S;
+            static_for<DEPTH>([&](auto k) {
+                if ((int)k < count) ring[k].load(row0 + (ptrdiff_t)k * row_stride);
+            });
+            pipelined<DEPTH>(count, [&](auto k, int j, auto checked) {
+                const FwdRow<SPL> row = ring[k];
+                if (!checked || j + DEPTH < count) ring[k].load(row0 + (ptrdiff_t)(j + DEPTH) * row_stride);
+                if (live) {
+                    FloatRun<SPL> mine;
+#pragma unroll
+                    for (int i = 0; i < SPL; ++i) mine.v[i] = f[i];
+                    mine.store(p0p + (size_t)j * S);
+                }
+                block_barrier_lds();
+                const float p0 = vecF[g][buf][q], p1 = vecF[g][buf][q + Q];
+                const float p2 = vecF[g][buf][q + 2 * Q], p3 = vecF[g][buf][q + 3 * Q];
+                fwd_update<0, SPL, M>(f, p0, p1, p2, p3, row, stay, logtab);
+                buf ^= 1;
+                FloatRun<SPL> mine;
+#pragma unroll
+                for (int i = 0; i < SPL; ++i) mine.v[i] = f[i];
+                mine.store(&vecF[g][buf][s0]);
+            });
+        };
+        const int warm = MODE == OFK_SCAN_TWO_TIER ? (cnt1 < kWarmup ? cnt1 : kWarmup) : 0;
+        if constexpr (MODE == OFK_SCAN_TWO_TIER) sweep1(std::integral_constant<int, OFK_SCAN_PRECISE>{}, 0, warm);
+        sweep1(std::integral_constant<int, MODE>{}, warm, cnt1 - warm);
+        for (int x = cnt1; x < T - H; ++x) block_barrier_lds();  // the backward lanes' extra step
+
+        // middle: shift = max_s(fwd[H][s] + bwd[H][s]) - 10
+        __syncthreads();
+        {
+            const int bbuf = (T - H) & 1;  // where the backward lanes left bwd[H]
+            FloatRun<SPL> bh;
+            bh.load(&vecB[g][bbuf][s0]);
+            float m = f[0] + bh.v[0];
+#pragma unroll
+            for (int i = 1; i < SPL; ++i) m = fmaxf(m, f[i] + bh.v[i]);
+            m = group_max<64>(m);
+            if ((tid & 63) == 0) part[g][1][0][wave] = m;
+            block_barrier_lds();
+            m = part[g][1][0][0];
+#pragma unroll
+            for (int w = 1; w < RW; ++w) m = fmaxf(m, part[g][1][0][w]);
+            if (l == 0) shift_of[g] = m - 10.0f;
+            block_barrier_lds();
+        }
+        const float shift = shift_of[g];
+
+        // phase 2: rows t = H .. T
+        const int cnt2 = T - H + 1;
+        int pb = 1;  // parity 0 of part[][1] was used for the maximum just now
+        {
+            const _Float16 *row0 = sp + (ptrdiff_t)H * row_stride;
+            const float *b0 = bp + (size_t)H * S;
+            float *p0p = pp + (size_t)H * S;
+            FloatRun<SPL> bring[DEPTH];
+            static_for<DEPTH>([&](auto k) {
+                if ((int)k < cnt2 - 1) ring[k].load(row0 + (ptrdiff_t)k * row_stride);
+                if ((int)k < cnt2) bring[k].load(b0 + (size_t)k * S);
+            });
+            pipelined<DEPTH, 1>(cnt2, [&](auto k, int j, auto checked) {
+                const FwdRow<SPL> row = ring[k];
+                const FloatRun<SPL> bw = bring[k];
+                if (!checked || j + DEPTH < cnt2 - 1) ring[k].load(row0 + (ptrdiff_t)(j + DEPTH) * row_stride);
+                if (!checked || j + DEPTH < cnt2) bring[k].load(b0 + (size_t)(j + DEPTH) * S);
+                FloatRun<SPL> e;
+                float total = 0.f;
+#pragma unroll
+                for (int i = 0; i < SPL; ++i) {
+                    e.v[i] = __builtin_amdgcn_exp2f(((f[i] + bw.v[i]) - shift) * kLog2e);
+                    total += e.v[i];
+                }
+                total = group_sum<64>(total);
+                if ((tid & 63) == 0) part[g][1][pb][wave] = total;
+                block_barrier_lds();
+                total = part[g][1][pb][0];
+#pragma unroll
+                for (int w = 1; w < RW; ++w) total += part[g][1][pb][w];
+                pb ^= 1;
+                const float inv = __builtin_amdgcn_rcpf(total);
+#pragma unroll
+                for (int i = 0; i < SPL; ++i) e.v[i] *= inv;
+                if (live) e.store(p0p + (size_t)j * S);
+                if (!checked || j + 1 < cnt2) {
+                    const float p0 = vecF[g][buf][q], p1 = vecF[g][buf][q + Q];
+                    const float p2 = vecF[g][buf][q + 2 * Q], p3 = vecF[g][buf][q + 3 * Q];
+                    fwd_update<0, SPL, MODE>(f, p0, p1, p2, p3, row, stay, logtab);
+                    buf ^= 1;
+                    FloatRun<SPL> mine;
+#pragma unroll
+                    for (int i = 0; i < SPL; ++i) mine.v[i] = f[i];
+                    mine.store(&vecF[g][buf][s0]);
+                }
+            });
+        }
+    }
+}
+
+const LogSeries kSeries = {OFA_LOG_SERIES, OFA_EXP_COEFS};
 
 template <int S, int SPL, int DEPTH>
-int launch_bwd(const void *scores, float *bwd, int T, int N, float stay, hipStream_t st) {
+int launch_bwd(int mode, const void *scores, float *bwd, int T, int N, float stay, hipStream_t st) {
     using Sh = Shape<S, SPL>;
-    const int blocks = (N + Sh::kChunks - 1) / Sh::kChunks;
-    if (g_scan_fast)
-        hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, false>), dim3(blocks), dim3(Sh::kThreads), 0, st,
-                           static_cast<const _Float16 *>(scores), bwd, T, N, stay, kSeries);
-    else
-        hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, true>), dim3(blocks), dim3(Sh::kThreads), 0, st,
-                           static_cast<const _Float16 *>(scores), bwd, T, N, stay, kSeries);
+    const dim3 grid((N + Sh::kChunks - 1) / Sh::kChunks), block(Sh::kThreads);
+    const _Float16 *sc = static_cast<const _Float16 *>(scores);
+    switch (mode) {
+        case OFK_SCAN_TWO_TIER:
+            hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, OFK_SCAN_TWO_TIER>), grid, block, 0, st, sc, bwd, T, N, stay, kSeries);
+            break;
+        case OFK_SCAN_PRECISE:
+            hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, OFK_SCAN_PRECISE>), grid, block, 0, st, sc, bwd, T, N, stay, kSeries);
+            break;
+        case OFK_SCAN_FAST:
+            hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, OFK_SCAN_FAST>), grid, block, 0, st, sc, bwd, T, N, stay, kSeries);
+            break;
+        default: return OFK_BAD_ARGS;
+    }
     return (int)hipGetLastError();
 }
 
 template <int S, int SPL, int DEPTH>
-int launch_fwd(const void *scores, const float *bwd, float *post, int T, int N, float stay, hipStream_t st) {
+int launch_fwd(int mode, const void *scores, const float *bwd, float *post, int T, int N, float stay, hipStream_t st) {
     using Sh = Shape<S, SPL>;
-    const int blocks = (N + Sh::kChunks - 1) / Sh::kChunks;
-    if (g_scan_fast)
-        hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, false>), dim3(blocks), dim3(Sh::kThreads), 0, st,
-                           static_cast<const _Float16 *>(scores), bwd, post, T, N, stay, kSeries);
-    else
-        hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, true>), dim3(blocks), dim3(Sh::kThreads), 0, st,
-                           static_cast<const _Float16 *>(scores), bwd, post, T, N, stay, kSeries);
+    const dim3 grid((N + Sh::kChunks - 1) / Sh::kChunks), block(Sh::kThreads);
+    const _Float16 *sc = static_cast<const _Float16 *>(scores);
+    switch (mode) {
+        case OFK_SCAN_TWO_TIER:
+            hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, OFK_SCAN_TWO_TIER>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            break;
+        case OFK_SCAN_PRECISE:
+            hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, OFK_SCAN_PRECISE>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            break;
+        case OFK_SCAN_FAST:
+            hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, OFK_SCAN_FAST>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            break;
+        default: return OFK_BAD_ARGS;
+    }
+    return (int)hipGetLastError();
+}
+
+template <int S, int SPL, int DEPTH>
+int launch_fused(int mode, const void *scores, float *bwd, float *post, int T, int N, float stay, hipStream_t st) {
+    using Sh = FusedShape<S, SPL>;
+    const dim3 grid((N + Sh::kChunks - 1) / Sh::kChunks), block(Sh::kThreads);
+    const _Float16 *sc = static_cast<const _Float16 *>(scores);
+    switch (mode) {
+        case OFK_SCAN_TWO_TIER:
+            hipLaunchKernelGGL((scan_post_kernel<S, SPL, DEPTH, OFK_SCAN_TWO_TIER>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            break;
+        case OFK_SCAN_PRECISE:
+            hipLaunchKernelGGL((scan_post_kernel<S, SPL, DEPTH, OFK_SCAN_PRECISE>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            break;
+        case OFK_SCAN_FAST:
+            hipLaunchKernelGGL((scan_post_kernel<S, SPL, DEPTH, OFK_SCAN_FAST>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            break;
+        default: return OFK_BAD_ARGS;
+    }
     return (int)hipGetLastError();
 }
 
@@ -472,9 +926,10 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // with a barrier per step, so that size stops at 2.
 // The backward sweep of the smaller models measures faster with two waves per SIMD
 // (hac, 512 chunks: 1.29 ms against 1.33 ms; 0.56 against 0.68 ms with hardware exp/log).
-int states_per_lane(int S, int N, bool backward) {
+// `forced` = 4, 2 or 1 overrides the choice (0 = choose).
+int states_per_lane(int S, int N, bool backward, int forced) {
     const int min_spl = S >= 1024 ? 2 : 1;
-    if (g_scan_spl == 4 || g_scan_spl == 2 || g_scan_spl == 1) return g_scan_spl < min_spl ? min_spl : g_scan_spl;
+    if (forced == 4 || forced == 2 || forced == 1) return forced < min_spl ? min_spl : forced;
     const long wanted = (backward && S <= 256) ? 2048 : 1024;
     for (int spl = 4; spl > min_spl; spl >>= 1) {
         const long waves = ((long)N * (S / spl) + 63) / 64;
@@ -485,35 +940,82 @@ int states_per_lane(int S, int N, bool backward) {
 
 }  // namespace
 
-extern "C" void ofk_set_scan_fast(int on) { g_scan_fast = on; }
-extern "C" void ofk_set_scan_states_per_lane(int spl) { g_scan_spl = spl; }
-
+#ifndef OFK_DEPTH
+#define OFK_DEPTH 8
+#endif
+#ifndef OFK_DEPTH_1024
+#define OFK_DEPTH_1024 6
+#endif
 #define OFK_DISPATCH(BACKWARD, LAUNCH, ...)                                                    \
-    switch (state_len * 8 + states_per_lane(1 << (2 * state_len), N, BACKWARD)) {             \
-        case 3 * 8 + 4: return LAUNCH<64, 4, 8>(__VA_ARGS__);                          \
-        case 3 * 8 + 2: return LAUNCH<64, 2, 8>(__VA_ARGS__);                          \
-        case 3 * 8 + 1: return LAUNCH<64, 1, 8>(__VA_ARGS__);                          \
-        case 4 * 8 + 4: return LAUNCH<256, 4, 8>(__VA_ARGS__);                         \
-        case 4 * 8 + 2: return LAUNCH<256, 2, 8>(__VA_ARGS__);                         \
-        case 4 * 8 + 1: return LAUNCH<256, 1, 8>(__VA_ARGS__);                         \
-        case 5 * 8 + 4: return LAUNCH<1024, 4, 6>(__VA_ARGS__);                        \
-        case 5 * 8 + 2: return LAUNCH<1024, 2, 6>(__VA_ARGS__);                        \
+    switch (state_len * 8 + states_per_lane(1 << (2 * state_len), N, BACKWARD, spl)) {        \
+        case 3 * 8 + 4: return LAUNCH<64, 4, OFK_DEPTH>(__VA_ARGS__);                          \
+        case 3 * 8 + 2: return LAUNCH<64, 2, OFK_DEPTH>(__VA_ARGS__);                          \
+        case 3 * 8 + 1: return LAUNCH<64, 1, OFK_DEPTH>(__VA_ARGS__);                          \
+        case 4 * 8 + 4: return LAUNCH<256, 4, OFK_DEPTH>(__VA_ARGS__);                         \
+        case 4 * 8 + 2: return LAUNCH<256, 2, OFK_DEPTH>(__VA_ARGS__);                         \
+        case 4 * 8 + 1: return LAUNCH<256, 1, OFK_DEPTH>(__VA_ARGS__);                         \
+        case 5 * 8 + 4: return LAUNCH<1024, 4, OFK_DEPTH_1024>(__VA_ARGS__);                        \
+        case 5 * 8 + 2: return LAUNCH<1024, 2, OFK_DEPTH_1024>(__VA_ARGS__);                        \
         default: return OFK_BAD_ARGS;                                                  \
     }
 
-extern "C" int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, float stay,
-                            void *stream) {
+// States per lane of the two-directional kernel: one direction of a chunk owns whole waves, so
+// 64 states need one state per lane; as many lanes as it takes to put four waves on every SIMD,
+// within the 1024 threads of a workgroup.
+static int fused_states_per_lane(int S, int N, int forced) {
+#ifdef OFK_FORCE_FUSED_SPL
+    if (S == 256) forced = OFK_FORCE_FUSED_SPL;
+#endif
+    const int min_spl = S >= 1024 ? 2 : 1, max_spl = S >= 256 ? 4 : 1;
+    if (forced == 4 || forced == 2 || forced == 1) return forced < min_spl ? min_spl : (forced > max_spl ? max_spl : forced);
+    for (int spl = max_spl; spl > min_spl; spl >>= 1) {
+        const long waves = (long)N * 2 * (S / spl) / 64;
+        if (waves >= 4096) return spl;
+    }
+    return min_spl;
+}
+
+#ifdef OFK_TIER_STATS
+extern "C" void ofk_tier_stats(unsigned long long *out, int reset) {
+    hipDeviceSynchronize();
+    hipMemcpyFromSymbol(out, HIP_SYMBOL(g_tier_stats), sizeof(unsigned long long) * 4);
+    if (reset) {
+        unsigned long long z[4] = {0, 0, 0, 0};
+        hipMemcpyToSymbol(HIP_SYMBOL(g_tier_stats), z, sizeof z);
+    }
+}
+#endif
+
+extern "C" int ofk_scan_posterior(const void *scores, float *bwd, float *post, int T, int N, int state_len,
+                                  float stay, int mode, int spl, void *stream) {
+    if (!scores || !bwd || !post || T < 1 || N < 1 || !aligned16(scores) || !aligned16(bwd) || !aligned16(post))
+        return OFK_BAD_ARGS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int S = 1 << (2 * state_len);
+    switch (state_len * 8 + (state_len >= 3 && state_len <= 5 ? fused_states_per_lane(S, N, spl) : 0)) {
+        case 3 * 8 + 1: return launch_fused<64, 1, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);
+        case 4 * 8 + 4: return launch_fused<256, 4, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);
+        case 4 * 8 + 2: return launch_fused<256, 2, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);
+        case 4 * 8 + 1: return launch_fused<256, 1, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);
+        case 5 * 8 + 4: return launch_fused<1024, 4, OFK_DEPTH_1024>(mode, scores, bwd, post, T, N, stay, st);
+        case 5 * 8 + 2: return launch_fused<1024, 2, OFK_DEPTH_1024>(mode, scores, bwd, post, T, N, stay, st);
+        default: return OFK_BAD_ARGS;
+    }
+}
+
+extern "C" int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, float stay, int mode,
+                            int spl, void *stream) {
     if (!scores || !bwd || T < 1 || N < 1 || !aligned16(scores) || !aligned16(bwd)) return OFK_BAD_ARGS;
     if (state_len < 3 || state_len > 5) return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    OFK_DISPATCH(true, launch_bwd, scores, bwd, T, N, stay, st)
+    OFK_DISPATCH(true, launch_bwd, mode, scores, bwd, T, N, stay, st)
 }
 
 extern "C" int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N,
-                                 int state_len, float stay, void *stream) {
+                                 int state_len, float stay, int mode, int spl, void *stream) {
     if (!scores || !bwd || !post || T < 1 || N < 1 || !aligned16(scores) || !aligned16(bwd) || !aligned16(post))
         return OFK_BAD_ARGS;
     if (state_len < 3 || state_len > 5) return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    OFK_DISPATCH(false, launch_fwd, scores, bwd, post, T, N, stay, st)
+    OFK_DISPATCH(false, launch_fwd, mode, scores, bwd, post, T, N, stay, st)
 }

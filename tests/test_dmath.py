@@ -24,6 +24,8 @@ def lib(tmp_path_factory):
     L.max_abs_err_log_tab.argtypes = [fp, C.c_long]
     L.lse5_mismatches.restype = C.c_long
     L.lse5_mismatches.argtypes = [fp, C.c_long]
+    L.two_tier_wrongly_settled.restype = C.c_long
+    L.two_tier_wrongly_settled.argtypes = [fp, C.c_long, C.POINTER(C.c_long), C.POINTER(C.c_long)]
     return L
 
 
@@ -68,3 +70,30 @@ def test_lse5_reproduces_the_libm_roundings(lib, centre, spread):
     rng = np.random.default_rng(int(abs(centre)) + 7)
     v = (centre + spread * rng.standard_normal((1000000, 5))).astype(np.float32)
     assert lib.lse5_mismatches(fptr(v), v.shape[0]) == 0
+
+
+@pytest.mark.parametrize("centre,spread,max_open", [(0.0, 3.0, 1.0), (100.0, 3.0, 0.25), (700.0, 3.0, 0.03),
+                                                    (3000.0, 3.0, 0.008), (5900.0, 3.0, 0.004), (5900.0, 40.0, 0.002),
+                                                    (48000.0, 30.0, 0.0003), (-3000.0, 0.3, 0.009), (-5000.0, 3.0, 0.004)])
+def test_two_tier_estimate_is_never_wrongly_settled(lib, centre, spread, max_open):
+    """the fp32 estimate of the scan update declares itself settled only where it equals the libm
+    result; the fraction left to the double arithmetic shrinks as an ulp of the values grows.
+    (Host build: libm's exp2f/log2f stand in for v_exp_f32/v_log_f32, whose measured error bounds
+    are the larger ones and are what the bound in dmath.h budgets for.)"""
+    rng = np.random.default_rng(int(abs(centre)) + 11)
+    v = (centre + spread * rng.standard_normal((400000, 5))).astype(np.float32)
+    unsettled, mismatches = C.c_long(), C.c_long()
+    wrong = lib.two_tier_wrongly_settled(fptr(v), v.shape[0], C.byref(unsettled), C.byref(mismatches))
+    assert wrong == 0 and mismatches.value == 0
+    assert unsettled.value <= max_open * v.shape[0]
+
+
+def test_two_tier_special_values_are_left_to_the_double_arithmetic(lib):
+    """results that are zero, a power of two or tiny never count as settled"""
+    cases = np.array([[0.0, -90.0, -90.0, -90.0, -90.0],      # exactly 0 + log(1 + tiny)
+                      [4096.0, 3000.0, 3000.0, 3000.0, 3000.0],  # a power of two
+                      [1e-3, -1.0, -2.0, -3.0, -4.0],
+                      [-2.5, -2.5, -2.5, -2.5, -2.5]], np.float32)
+    unsettled, mismatches = C.c_long(), C.c_long()
+    wrong = lib.two_tier_wrongly_settled(fptr(cases), cases.shape[0], C.byref(unsettled), C.byref(mismatches))
+    assert wrong == 0 and mismatches.value == 0 and unsettled.value == cases.shape[0]
