@@ -156,6 +156,29 @@ OFA_HD double log_1to5_tab(float s, const LogCell *table, const double *series) 
     return __builtin_fma((double)k, kLn2, lu);
 }
 
+// The same logarithm with the table cell (and the power of two) taken from an approximation
+// `near` of s, |near / s - 1| < 2^-18, so that the cell can be fetched before s is known: with k the
+// exponent of `near` and c its cell, ln s = k ln2 + ln c + log1p(s 2^-k / c - 1), and the argument of
+// log1p stays within 1/64 + 2^-17 in magnitude whichever side of a cell (or binade) boundary s itself
+// falls on: the ninth power, the first one the series drops, stays below 2^-56.
+OFA_HD LogCell log_cell_near(float near, const LogCell *table) { return table[(bits_of(near) >> 18) & 31u]; }
+OFA_HD double log_1to5_with_cell(float s, float near, LogCell c, const double *series) {
+    const int k = (int)(bits_of(near) >> 23) - 127;
+    const double u = __builtin_ldexp((double)s, -k);
+    const double r = __builtin_fma(u, c.inv, -1.0);
+    double q = series[0];
+    q = __builtin_fma(q, r, series[1]);
+    q = __builtin_fma(q, r, series[2]);
+    q = __builtin_fma(q, r, series[3]);
+    q = __builtin_fma(q, r, series[4]);
+    q = __builtin_fma(q, r, series[5]);
+    q = __builtin_fma(q, r, -0.5);
+    q = __builtin_fma(q, r, 1.0);
+    const double lu = __builtin_fma(q, r, c.lnc);
+    const double kLn2 = 0.69314718055994530942;
+    return __builtin_fma((double)k, kLn2, lu);
+}
+
 // RN32(m + ln s) as the CPU path forms it: the sum in double, one rounding.  ln 1 is exactly 0 on
 // the CPU path; the table logarithm returns about 1e-18 there, which would show in a result whose
 // m is zero.
@@ -224,6 +247,7 @@ OFA_HD float log2_hw(float x) {
 
 struct Lse5Estimate {
     float value;
+    float sum;  // the fp32 estimate of the sum of exponentials, within 1e-6 (relative) of the CPU path's
     bool settled;
 };
 OFA_HD Lse5Estimate lse5_estimate(float v0, float v1, float v2, float v3, float v4, float m) {
@@ -233,13 +257,15 @@ OFA_HD Lse5Estimate lse5_estimate(float v0, float v1, float v2, float v3, float 
     s += exp2_hw((v2 - m) * kLog2e);
     s += exp2_hw((v3 - m) * kLog2e);
     s += exp2_hw((v4 - m) * kLog2e);
+    const float kEps0 = 6.35e-7f, kEps1 = 0.65e-7f;
     const float l2 = log2_hw(s);
     Lse5Estimate e;
+    e.sum = s;
     e.value = __builtin_fmaf(l2, kLn2, m);
     const float rho = __builtin_fmaf(l2, kLn2, -(e.value - m));
     const uint32_t rb = bits_of(e.value);
     const float h = float_of((rb & 0x7f800000u) - (24u << 23));  // negative or huge-negative below 2^-102
-    const float eps = __builtin_fmaf(float_of(bits_of(s) & 0x7f800000u), 0.65e-7f, 6.35e-7f);
+    const float eps = __builtin_fmaf(float_of(bits_of(s) & 0x7f800000u), kEps1, kEps0);
     e.settled = (h - __builtin_fabsf(rho) > eps) && (rb & 0x007fffffu) != 0;
     return e;
 }

@@ -133,8 +133,14 @@ struct LogArgs {
 __device__ unsigned long long g_tier_stats[4];  // wave-level calls, calls with unsettled lanes, trips, unsettled lanes
 #endif
 
-__device__ __forceinline__ float resolve_unsettled(float value, bool unsettled, float v0, float v1, float v2, float v3,
-                                                   float v4, float m, const LogArgs &logtab) {
+#ifdef OFK_TIER_STATS
+// build with -DOFK_TIER_STATS to count, per wave-level update of the two-tier scans: updates, updates
+// with unsettled lanes, second-tier trips, unsettled lanes (read with ofk_tier_stats)
+__device__ unsigned long long g_tier_stats[4];
+#endif
+
+__device__ __forceinline__ float resolve_unsettled(float value, float sum, bool unsettled, float v0, float v1, float v2,
+                                                   float v3, float v4, float m, const LogArgs &logtab) {
     uint64_t mask = __builtin_amdgcn_ballot_w64(unsettled);
 #ifdef OFK_TIER_STATS
     if ((threadIdx.x & 63) == 0) {
@@ -153,17 +159,20 @@ __device__ __forceinline__ float resolve_unsettled(float value, bool unsettled, 
         if ((unsigned)rank < 8u) {
             float *slot = logtab.lanes + 8 * rank;
             *reinterpret_cast<float4 *>(slot) = make_float4(v0 - m, v1 - m, v2 - m, v3 - m);
-            *reinterpret_cast<float2 *>(slot + 4) = make_float2(v4 - m, m);
+            *reinterpret_cast<float4 *>(slot + 4) = make_float4(v4 - m, m, sum, 0.f);
         }
-        chunk_sync<false>();
-        const float x = logtab.lanes[lane];
-        chunk_sync<false>();  // the next trip (or call) of this wave writes the slots again
+        const float x = logtab.lanes[lane];  // LDS operations of one wave complete in order
+        // lane 8q+4 will take the logarithm: its table cell is fetched now, chosen with the estimate
+        // of the sum (two lanes up), and arrives while the exponentials are evaluated
+        const float near = dpp<0x102>(x);  // row_shl:2
+        const ofa::LogCell cell = ofa::log_cell_near(near, logtab.cells);
         const double e = ofa::exp_ldexp((double)x, logtab.expc);
         float s = (float)e;
 #pragma unroll
         for (int k = 0; k < 4; ++k) s = (float)((double)dpp<0x111>(s) + e);  // row_shr:1: the sum so far, from the lane below
         const float m_of_group = dpp<0x101>(x);  // row_shl:1: lane 8q+4 reads m from lane 8q+5
-        const float r = ofa::add_log_rounded(m_of_group, s, logtab.cells, logtab.series);
+        float r = (float)((double)m_of_group + ofa::log_1to5_with_cell(s, near, cell, logtab.series));
+        r = s == 1.0f ? m_of_group : r;  // ln 1 = 0 exactly, as on the CPU path
         const float mine = __int_as_float(__builtin_amdgcn_ds_bpermute((8 * (rank & 7) + 4) << 2, __float_as_int(r)));
         if ((unsigned)rank < 8u) value = mine;
         rank -= 8;
@@ -173,10 +182,18 @@ __device__ __forceinline__ float resolve_unsettled(float value, bool unsettled, 
     return value;
 }
 
+// maximum of three in one instruction (the operands are never NaN here; fmaxf would first quiet
+// each operand that comes out of inline assembly with an extra instruction)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // max + log(sum_i exp(v_i - max)), sum taken in the order v0..v4
 template <int MODE>
 __device__ __forceinline__ float lse5(float v0, float v1, float v2, float v3, float v4, const LogArgs &logtab) {
-    const float m = fmaxf(fmaxf(fmaxf(v0, v1), v2), fmaxf(v3, v4));
+    const float m = max3(max3(v0, v1, v2), v3, v4);
     if constexpr (MODE == OFK_SCAN_PRECISE) {
         return ofa::lse5_cpu_rounding_tab(v0, v1, v2, v3, v4, m, logtab.cells, logtab.series, logtab.expc);
     } else if constexpr (MODE == OFK_SCAN_TWO_TIER) {
@@ -186,7 +203,7 @@ __device__ __forceinline__ float lse5(float v0, float v1, float v2, float v3, fl
 #elif defined(OFK_EXPERIMENT_BALLOT_ONLY)
         return __builtin_amdgcn_ballot_w64(!e.settled) == 0x123456789ull ? m : e.value;
 #else
-        return resolve_unsettled(e.value, !e.settled, v0, v1, v2, v3, v4, m, logtab);
+        return resolve_unsettled(e.value, e.sum, !e.settled, v0, v1, v2, v3, v4, m, logtab);
 #endif
     } else {
         float s = __builtin_amdgcn_exp2f((v0 - m) * kLog2e);
@@ -612,21 +629,28 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
     if (!live) n = N - 1;
 
     const int H = T / 2;  // forward: rows 0..H-1 in phase 1, H..T in phase 2
+    // Addresses are a base that is the same for the whole workgroup (kept in scalar registers and
+    // stepped from row to row by scalar additions) plus a 32-bit offset of the lane that never changes.
     const ptrdiff_t row_stride = (ptrdiff_t)N * 4 * S;  // fp16 elements between time steps
-    const size_t chunk_off = (size_t)n * (size_t)(T + 1) * S;
+    const int first_chunk = blockIdx.x * Sh::kChunks;
+    const unsigned g_eff = (unsigned)(n - first_chunk);  // chunk within the group (dead lanes repeat the last chunk)
+    const _Float16 *const sc_blk = scores + (size_t)first_chunk * 4 * S;
+    const size_t blk_off = (size_t)first_chunk * (size_t)(T + 1) * S;
+    float *const bwd_blk = bwd + blk_off;
+    float *const post_blk = post + blk_off;
+    const unsigned chunk_rows = g_eff * (unsigned)(T + 1) * S;
 
     if (!forward) {
         // ------------------------------ backward lanes ------------------------------
         const int r = l / H4, c0 = (l % H4) * SPL;  // own states: r + (c0 + i) * Q
-        const _Float16 *sp = scores + (size_t)n * 4 * S + 16 * r + c0;
-        float *out = bwd + chunk_off + r + c0 * Q;
-        float *pp = post + chunk_off + r + c0 * Q;
+        const unsigned sc_lane = g_eff * 4 * S + 16 * r + c0;
+        const unsigned st_lane = chunk_rows + r + c0 * Q;
         float a[SPL];
 #pragma unroll
         for (int i = 0; i < SPL; ++i) {
             a[i] = 0.f;
             vecB[g][0][r + (c0 + i) * Q] = 0.f;
-            if (live) out[(size_t)T * S + i * Q] = 0.f;
+            if (live) bwd_blk[(size_t)T * S + st_lane + i * Q] = 0.f;
         }
         int buf = 0;
         BwdRow<SPL> ring[DEPTH];
@@ -637,14 +661,20 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
         const int cnt1 = T - H;
         auto sweep1 = [&](auto mode, int first, int count) {
             constexpr int M = decltype(mode)::value;
-            const _Float16 *row0 = sp + (ptrdiff_t)(T - 1 - first) * row_stride;
-            float *o0 = out + (ptrdiff_t)(T - 1 - first) * S;
+            const _Float16 *pre = sc_blk + (ptrdiff_t)(T - 1 - first) * row_stride;  // next row to fetch
+            float *orow = bwd_blk + (ptrdiff_t)(T - 1 - first) * S;
             static_for<DEPTH>([&](auto k) {
-                if ((int)k < count) ring[k].load(row0 - (ptrdiff_t)k * row_stride);
+                if ((int)k < count) {
+                    ring[k].load(pre + sc_lane);
+                    pre -= row_stride;
+                }
             });
             pipelined<DEPTH>(count, [&](auto k, int j, auto checked) {
                 const BwdRow<SPL> row = ring[k];
-                if (!checked || j + DEPTH < count) ring[k].load(row0 - (ptrdiff_t)(j + DEPTH) * row_stride);
+                if (!checked || j + DEPTH < count) {
+                    ring[k].load(pre + sc_lane);
+                    pre -= row_stride;
+                }
                 block_barrier_lds();
                 const float4 nx = *reinterpret_cast<const float4 *>(&vecB[g][buf][4 * r]);
                 bwd_update<0, SPL, M>(a, nx, row, stay, logtab);
@@ -653,8 +683,9 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                 for (int i = 0; i < SPL; ++i) vecB[g][buf][r + (c0 + i) * Q] = a[i];
                 if (live) {
 #pragma unroll
-                    for (int i = 0; i < SPL; ++i) o0[i * Q - (ptrdiff_t)j * S] = a[i];
+                    for (int i = 0; i < SPL; ++i) orow[st_lane + i * Q] = a[i];
                 }
+                orow -= S;
             });
         };
         const int warm = MODE == OFK_SCAN_TWO_TIER ? (cnt1 < kWarmup ? cnt1 : kWarmup) : 0;
@@ -672,15 +703,18 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
         int pb = 0;
         float e_prev[SPL];
         {
-            const _Float16 *row0 = sp + (ptrdiff_t)(H - 1) * row_stride;
-            float *o0 = out + (ptrdiff_t)(H - 1) * S;
-            float *p0 = pp + (ptrdiff_t)(H - 1) * S;
+            const _Float16 *pre = sc_blk + (ptrdiff_t)(H - 1) * row_stride;
+            const float *fpre = post_blk + (ptrdiff_t)(H - 1) * S;  // next parked row to fetch
+            float *orow = bwd_blk + (ptrdiff_t)(H - 1) * S;
+            float *prow = post_blk + (ptrdiff_t)H * S;  // row of the posterior that is stored next (one step late)
             float fring[DEPTH][SPL];
             static_for<DEPTH>([&](auto k) {
                 if ((int)k < cnt2) {
-                    ring[k].load(row0 - (ptrdiff_t)k * row_stride);
+                    ring[k].load(pre + sc_lane);
 #pragma unroll
-                    for (int i = 0; i < SPL; ++i) fring[k][i] = p0[i * Q - (ptrdiff_t)k * S];
+                    for (int i = 0; i < SPL; ++i) fring[k][i] = fpre[st_lane + i * Q];
+                    pre -= row_stride;
+                    fpre -= S;
                 }
             });
             pipelined<DEPTH>(cnt2, [&](auto k, int j, auto checked) {
@@ -689,9 +723,11 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
 #pragma unroll
                 for (int i = 0; i < SPL; ++i) fv[i] = fring[k][i];
                 if (!checked || j + DEPTH < cnt2) {
-                    ring[k].load(row0 - (ptrdiff_t)(j + DEPTH) * row_stride);
+                    ring[k].load(pre + sc_lane);
 #pragma unroll
-                    for (int i = 0; i < SPL; ++i) fring[k][i] = p0[i * Q - (ptrdiff_t)(j + DEPTH) * S];
+                    for (int i = 0; i < SPL; ++i) fring[k][i] = fpre[st_lane + i * Q];
+                    pre -= row_stride;
+                    fpre -= S;
                 }
                 block_barrier_lds();
                 if (j > 0) {  // posterior of the previous row: its total is complete now
@@ -701,26 +737,28 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                     const float inv = __builtin_amdgcn_rcpf(total);
                     if (live) {
 #pragma unroll
-                        for (int i = 0; i < SPL; ++i) p0[i * Q - (ptrdiff_t)(j - 1) * S] = e_prev[i] * inv;
+                        for (int i = 0; i < SPL; ++i) prow[st_lane + i * Q] = e_prev[i] * inv;
                     }
                 }
+                prow -= S;
                 const float4 nx = *reinterpret_cast<const float4 *>(&vecB[g][buf][4 * r]);
                 bwd_update<0, SPL, MODE>(a, nx, row, stay, logtab);
                 buf ^= 1;
-                float total = 0.f;
+                float total;
 #pragma unroll
                 for (int i = 0; i < SPL; ++i) {
                     vecB[g][buf][r + (c0 + i) * Q] = a[i];
                     e_prev[i] = __builtin_amdgcn_exp2f(((fv[i] + a[i]) - shift) * kLog2e);
-                    total += e_prev[i];
+                    total = i ? total + e_prev[i] : e_prev[i];
                 }
                 total = group_sum<64>(total);
                 if ((tid & 63) == 0) part[g][0][pb][wave] = total;
                 pb ^= 1;
                 if (live) {
 #pragma unroll
-                    for (int i = 0; i < SPL; ++i) o0[i * Q - (ptrdiff_t)j * S] = a[i];
+                    for (int i = 0; i < SPL; ++i) orow[st_lane + i * Q] = a[i];
                 }
+                orow -= S;
             });
         }
         block_barrier_lds();
@@ -731,7 +769,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
             const float inv = __builtin_amdgcn_rcpf(total);
             if (live) {
 #pragma unroll
-                for (int i = 0; i < SPL; ++i) pp[i * Q] = e_prev[i] * inv;  // row 0
+                for (int i = 0; i < SPL; ++i) post_blk[st_lane + i * Q] = e_prev[i] * inv;  // row 0
             }
         }
         // the forward lanes take T - H + 1 barriers in phase 2, these took H + 1
@@ -739,9 +777,8 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
     } else {
         // ------------------------------ forward lanes ------------------------------
         const int s0 = SPL * l, q = s0 >> 2;  // own states s0 .. s0+SPL-1, all in quad q
-        const _Float16 *sp = scores + (size_t)n * 4 * S + 4 * s0;
-        const float *bp = bwd + chunk_off + s0;
-        float *pp = post + chunk_off + s0;
+        const unsigned sc_lane = g_eff * 4 * S + 4 * s0;
+        const unsigned st_lane = chunk_rows + s0;
         float f[SPL];
 #pragma unroll
         for (int i = 0; i < SPL; ++i) {
@@ -756,20 +793,27 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
         const int cnt1 = H;
         auto sweep1 = [&](auto mode, int first, int count) {
             constexpr int M = decltype(mode)::value;
-            const _Float16 *row0 = sp + (ptrdiff_t)first * row_stride;
-            float *p0p = pp + (size_t)first * S;
+            const _Float16 *pre = sc_blk + (ptrdiff_t)first * row_stride;
+            float *prow = post_blk + (size_t)first * S;
             static_for<DEPTH>([&](auto k) {
-                if ((int)k < count) ring[k].load(row0 + (ptrdiff_t)k * row_stride);
+                if ((int)k < count) {
+                    ring[k].load(pre + sc_lane);
+                    pre += row_stride;
+                }
             });
             pipelined<DEPTH>(count, [&](auto k, int j, auto checked) {
                 const FwdRow<SPL> row = ring[k];
-                if (!checked || j + DEPTH < count) ring[k].load(row0 + (ptrdiff_t)(j + DEPTH) * row_stride);
+                if (!checked || j + DEPTH < count) {
+                    ring[k].load(pre + sc_lane);
+                    pre += row_stride;
+                }
                 if (live) {
                     FloatRun<SPL> mine;
 #pragma unroll
                     for (int i = 0; i < SPL; ++i) mine.v[i] = f[i];
-                    mine.store(p0p + (size_t)j * S);
+                    mine.store(prow + st_lane);
                 }
+                prow += S;
                 block_barrier_lds();
                 const float p0 = vecF[g][buf][q], p1 = vecF[g][buf][q + Q];
                 const float p2 = vecF[g][buf][q + 2 * Q], p3 = vecF[g][buf][q + 3 * Q];
@@ -810,25 +854,29 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
         const int cnt2 = T - H + 1;
         int pb = 1;  // parity 0 of part[][1] was used for the maximum just now
         {
-            const _Float16 *row0 = sp + (ptrdiff_t)H * row_stride;
-            const float *b0 = bp + (size_t)H * S;
-            float *p0p = pp + (size_t)H * S;
+            const _Float16 *pre = sc_blk + (ptrdiff_t)H * row_stride;
+            const float *bpre = bwd_blk + (size_t)H * S;
+            float *prow = post_blk + (size_t)H * S;
             FloatRun<SPL> bring[DEPTH];
             static_for<DEPTH>([&](auto k) {
-                if ((int)k < cnt2 - 1) ring[k].load(row0 + (ptrdiff_t)k * row_stride);
-                if ((int)k < cnt2) bring[k].load(b0 + (size_t)k * S);
+                if ((int)k < cnt2 - 1) ring[k].load(pre + sc_lane);
+                if ((int)k < cnt2) bring[k].load(bpre + st_lane);
+                pre += row_stride;
+                bpre += S;
             });
             pipelined<DEPTH, 1>(cnt2, [&](auto k, int j, auto checked) {
                 const FwdRow<SPL> row = ring[k];
                 const FloatRun<SPL> bw = bring[k];
-                if (!checked || j + DEPTH < cnt2 - 1) ring[k].load(row0 + (ptrdiff_t)(j + DEPTH) * row_stride);
-                if (!checked || j + DEPTH < cnt2) bring[k].load(b0 + (size_t)(j + DEPTH) * S);
+                if (!checked || j + DEPTH < cnt2 - 1) ring[k].load(pre + sc_lane);
+                if (!checked || j + DEPTH < cnt2) bring[k].load(bpre + st_lane);
+                pre += row_stride;
+                bpre += S;
                 FloatRun<SPL> e;
-                float total = 0.f;
+                float total;
 #pragma unroll
                 for (int i = 0; i < SPL; ++i) {
                     e.v[i] = __builtin_amdgcn_exp2f(((f[i] + bw.v[i]) - shift) * kLog2e);
-                    total += e.v[i];
+                    total = i ? total + e.v[i] : e.v[i];
                 }
                 total = group_sum<64>(total);
                 if ((tid & 63) == 0) part[g][1][pb][wave] = total;
@@ -840,7 +888,8 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                 const float inv = __builtin_amdgcn_rcpf(total);
 #pragma unroll
                 for (int i = 0; i < SPL; ++i) e.v[i] *= inv;
-                if (live) e.store(p0p + (size_t)j * S);
+                if (live) e.store(prow + st_lane);
+                prow += S;
                 if (!checked || j + 1 < cnt2) {
                     const float p0 = vecF[g][buf][q], p1 = vecF[g][buf][q + Q];
                     const float p2 = vecF[g][buf][q + 2 * Q], p3 = vecF[g][buf][q + 3 * Q];
@@ -982,6 +1031,17 @@ extern "C" void ofk_tier_stats(unsigned long long *out, int reset) {
     if (reset) {
         unsigned long long z[4] = {0, 0, 0, 0};
         hipMemcpyToSymbol(HIP_SYMBOL(g_tier_stats), z, sizeof z);
+    }
+}
+#endif
+
+#ifdef OFK_TIER_STATS
+extern "C" void ofk_tier_stats(unsigned long long *out, int reset) {
+    (void)hipDeviceSynchronize();
+    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_tier_stats), sizeof(unsigned long long) * 4);
+    if (reset) {
+        unsigned long long z[4] = {0, 0, 0, 0};
+        (void)hipMemcpyToSymbol(HIP_SYMBOL(g_tier_stats), z, sizeof z);
     }
 }
 #endif

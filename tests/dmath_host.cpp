@@ -34,6 +34,24 @@ double max_abs_err_log_tab(const float *s, long n) {
     return worst;
 }
 
+// largest absolute error of the logarithm whose table cell comes from a neighbour `near` of s
+// (s moved by up to `ulps` fp32 steps either way), against logl
+double max_abs_err_log_near(const float *s, long n, int ulps) {
+    ofa::LogCell table[32];
+    for (int i = 0; i < 32; ++i) table[i] = ofa::log_cell(i);
+    double worst = 0;
+    for (long i = 0; i < n; ++i) {
+        for (int d = -ulps; d <= ulps; d += (ulps > 0 ? ulps : 1)) {
+            const float near = ofa::float_of(ofa::bits_of(s[i]) + (uint32_t)d);
+            if (!(near >= 1.0f)) continue;
+            const double got = ofa::log_1to5_with_cell(s[i], near, ofa::log_cell_near(near, table), kSeries);
+            const double err = (double)fabsl((long double)got - logl((long double)s[i]));
+            if (err > worst) worst = err;
+        }
+    }
+    return worst;
+}
+
 // the CPU path's own arithmetic (libm exp/log in double, fp32 running sum)
 static float lse5_libm(const float v[5], float m) {
     float acc = 0.0f;

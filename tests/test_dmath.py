@@ -24,6 +24,8 @@ def lib(tmp_path_factory):
     L.max_abs_err_log_tab.argtypes = [fp, C.c_long]
     L.lse5_mismatches.restype = C.c_long
     L.lse5_mismatches.argtypes = [fp, C.c_long]
+    L.max_abs_err_log_near.restype = C.c_double
+    L.max_abs_err_log_near.argtypes = [fp, C.c_long, C.c_int]
     L.two_tier_wrongly_settled.restype = C.c_long
     L.two_tier_wrongly_settled.argtypes = [fp, C.c_long, C.POINTER(C.c_long), C.POINTER(C.c_long)]
     return L
@@ -60,6 +62,18 @@ def test_table_log_absolute_error_below_2_pow_minus_51(lib):
                         [1.0, 5.0, 2.0, 4.0, 1.015625, 1.9999999, 3.9999998,
                          np.nextafter(np.float32(1), np.float32(2))]]).astype(np.float32)
     assert lib.max_abs_err_log_tab(fptr(s), s.size) < 2.0 ** -51
+
+
+def test_log_with_a_cell_chosen_from_a_neighbour(lib):
+    """the second tier fetches the table cell with the fp32 estimate of the sum, which may lie a few
+    ulps away from the sum itself, on the other side of a cell or binade boundary"""
+    rng = np.random.default_rng(5)
+    edges = 1 + np.arange(0, 129) / 32.0  # cell boundaries of [1, 5]
+    s = np.concatenate([1 + 4 * rng.random(300000), edges, np.nextafter(edges.astype(np.float32), np.float32(9)),
+                        np.nextafter(edges.astype(np.float32), np.float32(0)), [2.0, 4.0, 1.9999999, 3.9999998]]).astype(np.float32)
+    s = s[(s >= 1) & (s <= 5)]
+    assert lib.max_abs_err_log_near(fptr(s), s.size, 0) < 2.0 ** -51
+    assert lib.max_abs_err_log_near(fptr(s), s.size, 40) < 2.0 ** -51  # 40 ulps: 5e-6 relative
 
 
 @pytest.mark.parametrize("centre,spread", [(0.0, 3.0), (37.0, 2.0), (5900.0, 4.0), (5900.0, 40.0), (48000.0, 30.0),
