@@ -100,6 +100,21 @@ void openfish_amd_beam_search(int T, int N, int C, const void *scores, int state
                               const openfish_gpubuf_t *gpubuf);
 
 /*
+ * The same beam search and traceback for callers that must not allocate device memory (code
+ * under HIP graph capture, tight serving loops): it has no counterpart in the reference.
+ * Instead of a gpubuf it uses a static array of the library in device memory (64 MiB of beam
+ * slots plus the log-sum-exp table, held by every GPU the library runs on until the process
+ * ends) and writes its results to caller-provided device buffers: states int32 [N][T] (the
+ * k-mer state of the traced path) and moves uint8 [N][T].  N * (T + 1) * 64 bytes must fit the
+ * 64 MiB (hac at T = 1666: N <= 628), otherwise the call prints an error and exits.  It calls no
+ * hipMalloc/hipFree; the first call on a device looks up the array's address and copies the
+ * 4.9 KB table into it.  All calls on one GPU share the array: calls that overlap in time race.
+ */
+void openfish_amd_beam_search_static(int T, int N, int C, const void *scores, int state_len,
+                                     const openfish_opt_t *options, const float *bwd, int32_t *states,
+                                     uint8_t *moves);
+
+/*
  * Per-block quality, base calls and phred string (reference src/beam_search.c:441-496
  * and generate_sequence_cpu src/beam_search.c:49-99).  Reads post, gpubuf->states and
  * gpubuf->moves; fills gpubuf->qual_data, base_probs, total_probs, sequence, qstring

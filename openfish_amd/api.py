@@ -81,6 +81,7 @@ _SIGS = {
     "openfish_amd_scan_posterior": (None, [_i, _i, _i, _vp, _i, _f, _i, _vp, _vp]),
     "openfish_amd_gpubuf_set_split_scans": (None, [_bufp, _i]),
     "openfish_amd_beam_search": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _bufp]),
+    "openfish_amd_beam_search_static": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _vp, _vp]),
     "openfish_amd_sequence": (None, [_i, _i, _i, _optp, _vp, _bufp]),
     "openfish_amd_decode_enqueue": (None, [_i, _i, _i, _vp, _i, _optp, _bufp]),
     "openfish_amd_decode_wait": (None, [_bufp, _pp, _pp, _pp]),
@@ -282,6 +283,12 @@ def openfish_amd_scan_posterior(T, N, Cc, scores_dev, state_len, stay_score, bwd
 
 def openfish_amd_beam_search(T, N, Cc, scores_dev, state_len, options, bwd_dev, gpubuf):
     _L.openfish_amd_beam_search(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), _ptr(bwd_dev), gpubuf.handle)
+
+
+def openfish_amd_beam_search_static(T, N, Cc, scores_dev, state_len, options, bwd_dev, states_dev, moves_dev):
+    """the beam search on the library's static scratch array: allocates nothing"""
+    _L.openfish_amd_beam_search_static(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), _ptr(bwd_dev),
+                                       _ptr(states_dev), _ptr(moves_dev))
 
 
 def openfish_amd_sequence(T, N, state_len, options, post_dev, gpubuf):

@@ -24,6 +24,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cfloat>
+#include <mutex>
 
 #include "kernels.h"
 
@@ -720,6 +721,60 @@ int launch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int
 }
 
 }  // namespace
+
+// ---------------------------------------------------------------------------------------------
+// The same search with its scratch memory (the persisted beam slots the traceback walks, and the
+// log-sum-exp table) in a static device array instead of buffers of a gpubuf: for callers that
+// must not allocate.  Every GPU the library runs on holds its own copy of the array until the
+// process ends; `scratch` below is only the host-side handle of it, the device address comes
+// from hipGetSymbolAddress, once per device.
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+constexpr size_t kStaticTableBytes = 8192;  // 612 doubles, rounded up
+static __device__ __align__(256) unsigned char scratch[kStaticTableBytes + OFK_STATIC_SLOT_BYTES];
+
+constexpr int kMaxDevices = 64;
+unsigned char *g_scratch_of[kMaxDevices];  // device address of `scratch` per device, once looked up
+std::mutex g_scratch_mutex;
+
+}  // namespace
+
+extern "C" int ofk_beam_search_static(const void *scores, const float *bwd, int32_t *states, uint8_t *moves, int T,
+                                      int N, int state_len, float log_beam_cut, float stay,
+                                      const double *lse_table_host, int flags, void *stream) {
+    if (!scores || !bwd || !states || !moves || !lse_table_host || T < 1 || N < 1) return OFK_BAD_ARGS;
+    if ((reinterpret_cast<uintptr_t>(scores) | reinterpret_cast<uintptr_t>(bwd)) & 15u) return OFK_BAD_ARGS;
+    if ((size_t)N * (size_t)(T + 1) * kW * sizeof(ofk_beam_slot_t) > (size_t)OFK_STATIC_SLOT_BYTES) return OFK_TOO_LARGE;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return OFK_BAD_ARGS;
+    unsigned char *base;
+    {
+        // set-up, once per device: the array's device address, and the table copied behind it
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_of[dev]) {
+            void *p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) return (int)e;
+            e = hipMemcpy(p, lse_table_host, sizeof(double) * OFK_LSE_DOUBLES, hipMemcpyHostToDevice);
+            if (e != hipSuccess) return (int)e;
+            g_scratch_of[dev] = static_cast<unsigned char *>(p);
+        }
+        base = g_scratch_of[dev];
+    }
+    // nothing in the array has to start at zero: the search writes every slot the traceback reads
+    ofk_beam_slot_t *beam = reinterpret_cast<ofk_beam_slot_t *>(base + kStaticTableBytes);
+    const double *lse_table = reinterpret_cast<const double *>(base);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (state_len) {
+        case 3: return launch_beam<64>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
+        case 4: return launch_beam<256>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
+        case 5: return launch_beam<1024>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
+        default: return OFK_BAD_ARGS;
+    }
+}
 
 extern "C" int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                                uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,

@@ -16,6 +16,7 @@ extern "C" {
 /* longest chunk in time steps: the sequence stage keeps 14 bytes per step in LDS (160 KB) */
 #define OFK_MAX_T 8192
 #define OFK_BAD_ARGS (-1)
+#define OFK_TOO_LARGE (-2)
 #define OFK_BEAM_WIDTH 32
 
 /* one persisted beam slot, 16 bit: state[9:0] | prev[14:10] | stay[15] */
@@ -52,6 +53,15 @@ int ofk_scan_posterior(const void *scores, float *bwd, float *post, int T, int N
 int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                     uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
                     const double *lse_table, int flags, void *stream);
+/* The same search with the beam slots and the table in a static device array of the library
+ * (OFK_STATIC_SLOT_BYTES of slots: N * (T + 1) * 64 bytes must fit, else OFK_TOO_LARGE and nothing
+ * is launched).  Allocates nothing; the first call on a device looks up the array's address and
+ * copies the 612 doubles at lse_table_host (host memory) into it.  Calls that overlap in time on
+ * one device share the array and race. */
+#define OFK_STATIC_SLOT_BYTES (64u << 20)
+int ofk_beam_search_static(const void *scores, const float *bwd, int32_t *states, uint8_t *moves, int T, int N,
+                           int state_len, float log_beam_cut, float stay, const double *lse_table_host, int flags,
+                           void *stream);
 /* flags bit 0: replay every stay/step merge one by one in CPU order (the path otherwise taken
  * only after a hash collision); results must not change.  For tests. */
 /* Phred characters run from '"' (34, q = 1) to 'S' (83, q = 50).  thr[j] is the smallest

@@ -533,6 +533,25 @@ void openfish_amd_beam_search(int T, int N, int C, const void *scores, int state
     HIP_OK(hipStreamSynchronize(0));
 }
 
+void openfish_amd_beam_search_static(int T, int N, int C, const void *scores, int state_len,
+                                     const openfish_opt_t *options, const float *bwd, int32_t *states,
+                                     uint8_t *moves) {
+    check_scores(T, N, C, scores, state_len, options);
+    if (!bwd || !states || !moves) die("beam_search_static: bwd, states and moves must be device pointers");
+    double tab[OFK_LSE_DOUBLES]; /* read by the first call on a device only */
+    build_lse_table(tab);
+    const int rc = ofk_beam_search_static(scores, bwd, states, moves, T, N, state_len, log_beam_cut(options),
+                                          options->blank_score, tab, 0, NULL);
+    if (rc == OFK_TOO_LARGE) {
+        fprintf(stderr, "openfish: beam_search_static: N * (T + 1) * 64 = %zu bytes of beam slots exceed the static "
+                        "scratch array of %u bytes; use openfish_amd_beam_search with a gpubuf\n",
+                (size_t)N * (size_t)(T + 1) * 64, (unsigned)OFK_STATIC_SLOT_BYTES);
+        exit(EXIT_FAILURE);
+    }
+    launch_ok(rc, "beam_search_static");
+    HIP_OK(hipStreamSynchronize(0));
+}
+
 void openfish_amd_sequence(int T, int N, int state_len, const openfish_opt_t *options, const float *post,
                            const openfish_gpubuf_t *gpubuf) {
     if (!options) die("options is NULL");

@@ -1,0 +1,47 @@
+"""The beam search entry point that allocates nothing (its scratch is a static device array of
+the library) against the entry point that works on a gpubuf, through the C-ABI: same states and
+moves, bit for bit, on two calls in a row, the second one smaller."""
+import numpy as np
+import pytest
+
+from openfish_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def api():
+    from openfish_amd import api as _api
+    if _api.device_count() < 1:
+        pytest.skip("no HIP device")
+    return _api
+
+
+def both_entry_points(api, state_len, T, N, seed, scale=None, **opt_kw):
+    S = 4 ** state_len
+    C = 4 * S
+    s16 = synth.crf_scores(T, N, state_len, seed=seed, chunk_scale=scale)
+    sc = api.upload_scores_to_hip(s16)
+    bwd = api.DeviceBuffer(4 * N * (T + 1) * S)
+    api.openfish_amd_bwd_scan(T, N, C, sc, state_len, 2.0, bwd)
+    opt = api.DECODER_INIT(**opt_kw)
+
+    gb = api.GpuBuf(T, N, state_len)
+    api.openfish_amd_beam_search(T, N, C, sc, state_len, opt, bwd, gb)
+    want_states, want_moves = gb.tensor("states"), gb.tensor("moves")
+
+    states, moves = api.DeviceBuffer(4 * N * T), api.DeviceBuffer(N * T)
+    states.fill(0xEE)
+    moves.fill(0xEE)
+    api.openfish_amd_beam_search_static(T, N, C, sc, state_len, opt, bwd, states, moves)
+    got_states, got_moves = states.to_host(np.int32, (N, T)), moves.to_host(np.uint8, (N, T))
+    assert np.array_equal(got_moves, want_moves)
+    assert np.array_equal(got_states, want_states)
+    assert got_moves[:, 0].all() and set(np.unique(got_moves)) <= {0, 1}
+
+
+def test_static_scratch_entry_point_matches_the_gpubuf_one_twice(api):
+    both_entry_points(api, 4, 400, 9, seed=71, scale=synth.stress_scale(9))
+    both_entry_points(api, 4, 150, 3, seed=72)  # smaller: the array still holds the first call's slots
+    both_entry_points(api, 3, 90, 5, seed=73, beam_cut=3.0)
+    both_entry_points(api, 5, 60, 2, seed=74)
