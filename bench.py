@@ -36,32 +36,36 @@ WORKLOADS = {
 }
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch in GB, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the plain
-# copy kernel's reading of the same counters (profiles/decode_*.md); keyed by workload and kernel
-MEASURED_TRAFFIC_GB = {
-    ("hac", 512, "bwd"): 2.621, ("hac", 512, "fwd_post"): 3.495, ("hac", 512, "beam"): 2.735,
-    ("hac", 512, "sequence"): 0.694,
-    ("fast", 512, "bwd"): 0.655, ("fast", 512, "fwd_post"): 0.874, ("fast", 512, "beam"): 0.769,
-    ("fast", 512, "sequence"): 0.291,
-    ("sup", 256, "bwd"): 5.242, ("sup", 256, "fwd_post"): 7.013, ("sup", 256, "beam"): 5.299,
-    ("sup", 256, "sequence"): 0.332,
-    ("hac_stress", 1024, "bwd"): 5.242, ("hac_stress", 1024, "fwd_post"): 7.004,
-    ("hac_stress", 1024, "beam"): 5.502, ("hac_stress", 1024, "sequence"): 1.830,
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
 
-def algorithmic_bytes(state_len, T, N):
-    """bytes each kernel has to move at least once, per launch"""
+def measured_traffic(workload, N, columns, kernel):
+    """HBM bytes per launch of one kernel as rocprofv3 counted them (FETCH_SIZE + WRITE_SIZE, each
+    scaled by the plain copy kernel's reading of the same counter): read from the summary the
+    profiling script wrote (profiles/traffic.json); None where that run has not been made"""
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            table = json.load(fh)
+    except (OSError, ValueError):
+        return None
+    entry = table.get("%s_n%d_c%d" % (workload, N, columns), {}).get(kernel)
+    return None if entry is None else int(round(entry["hbm_bytes"]))
+
+
+def algorithmic_bytes(state_len, T, N, columns=4):
+    """bytes each kernel has to move at least once, per launch (C = columns * S scores per time step)"""
     S = 4 ** state_len
-    C = 4 * S
+    C = columns * S
     scores = T * C * 2
     vec = (T + 1) * S * 4
-    return {
+    need = {
         "bwd": N * (scores + vec),                    # read scores, write bwd
         "fwd_post": N * (scores + 2 * vec),           # read scores + bwd, write post
         "beam": N * (scores + T * S * 4 + (T + 1) * 32 * 2 * 2 + 5 * T),  # rows, beam slots out+in, states+moves
         "sequence": N * (9 * 4 * T + 5 * T + 16 * T + 8 * T + 2 * T),  # gathers, states/moves, qual, probs, text
     }
+    need["scan"] = need["bwd"] + need["fwd_post"]     # both scans + posterior as one kernel: the same minimum
+    return need
 
 
 def cpu_baseline(s16, state_len, opt_kw, sample_chunks):
@@ -122,6 +126,28 @@ def rotary_bench(a):
         "cpu_baseline": None}))
 
 
+def timed_decodes(api, gpubuf, call_args, steps):
+    """`steps` blocking decodes: wall-clock ms per call and the mean device time of every stage"""
+    per_stage = {k: [] for k in api.STAGES}
+    api.lib().openfish_amd_sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        api.openfish_decode_gpu_discard(*call_args, gpubuf)
+        for k, v in gpubuf.timings().items():
+            per_stage[k].append(v)
+    api.lib().openfish_amd_sync()
+    ms = 1e3 * (time.perf_counter() - t0) / steps
+    return ms, {k: statistics.mean(v) for k, v in per_stage.items()}
+
+
+def scan_stage(need, mean):
+    """scans + posterior: one kernel (`scan`) or the two split kernels (`bwd`, `fwd_post`)"""
+    ms = mean["scan"] + mean["bwd"] + mean["fwd_post"]
+    gbs = need["scan"] / 1e9 / (ms / 1e3)
+    return {"ms": round(ms, 4), "algorithmic_GB": round(need["scan"] / 1e9, 4), "GBps": round(gbs, 1),
+            "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -129,11 +155,17 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="hac", choices=sorted(WORKLOADS) + ["rotary"])
     ap.add_argument("--chunks", type=int, default=0, help="override N")
+    ap.add_argument("--columns", type=int, default=4, choices=(4, 5),
+                    help="scores per state and time step: 4 (what the reference consumes) or 5 (a blank column first, "
+                         "C = 5 * 4^state_len as the network emits it)")
     ap.add_argument("--scan-mode", default="two_tier", choices=("two_tier", "precise", "fast"))
+    ap.add_argument("--split-scans", action="store_true",
+                    help="backward scan, then forward scan beside the beam search, instead of both scans as one kernel")
     ap.add_argument("--cpu-sample", type=int, default=512, help="chunks timed on the CPU path (0 = skip; capped at N)")
     ap.add_argument("--seed", type=int, default=20251125)
     ap.add_argument("--alt-steps", type=int, default=3,
-                    help="extra timed calls with the hardware-exp scan arithmetic, reported beside the main result (0 = skip)")
+                    help="extra timed calls per side measurement (split scans, hardware-exp scans), reported beside the "
+                         "main result (0 = skip)")
     ap.add_argument("--overlap-steps", type=int, default=5,
                     help="calls per gpubuf of the two-batches-in-flight side measurement (0 = skip)")
     ap.add_argument("--copy-mib", type=int, default=1024,
@@ -156,14 +188,18 @@ def main():
     if a.chunks:
         N = a.chunks
     S = 4 ** state_len
-    C = 4 * S
+    C = a.columns * S
     scale = synth.stress_scale(N) if stress else None
-    s16 = synth.crf_scores(T, N, state_len, seed=a.seed, chunk_scale=scale, threads=16)
+    made = synth.crf_scores(T, N, state_len, seed=a.seed, chunk_scale=scale, threads=16, five_columns=a.columns == 5)
+    s16, device_input = (made[0], made[1]) if a.columns == 5 else (made, made)  # s16: the four-column view
 
     opt = api.DECODER_INIT(q_scale=q_scale, q_shift=q_shift)
-    scores = api.upload_scores_to_hip(s16)
+    scores = api.upload_scores_to_hip(device_input)
+    del made, device_input
     gpubuf = api.GpuBuf(T, N, state_len)
     gpubuf.set_scan_mode(a.scan_mode)
+    gpubuf.set_split_scans(a.split_scans)
+    call = (T, N, C, scores, state_len, opt)
 
     if a.calibrate_copy:
         nbytes = a.calibrate_copy << 20
@@ -174,53 +210,45 @@ def main():
         dst.free()
 
     for _ in range(a.warmup):
-        api.openfish_decode_gpu_discard(T, N, C, scores, state_len, opt, gpubuf)
-    api.lib().openfish_amd_sync()
-    per_stage = {k: [] for k in api.STAGES}
-    t0 = time.perf_counter()
-    for _ in range(a.steps):
-        api.openfish_decode_gpu_discard(T, N, C, scores, state_len, opt, gpubuf)
-        for k, v in gpubuf.timings().items():
-            per_stage[k].append(v)
-    api.lib().openfish_amd_sync()
-    wall = time.perf_counter() - t0
-    ms_per_step = 1e3 * wall / a.steps
+        api.openfish_decode_gpu_discard(*call, gpubuf)
+    ms_per_step, mean = timed_decodes(api, gpubuf, call, a.steps)
 
-    need = algorithmic_bytes(state_len, T, N)
+    need = algorithmic_bytes(state_len, T, N, a.columns)
     stages = {}
-    for k in ("bwd", "fwd_post", "beam", "sequence"):
-        ms = statistics.mean(per_stage[k])
-        stages[k] = {"ms": round(ms, 4), "algorithmic_GB": round(need[k] / 1e9, 4),
-                     "GBps": round(need[k] / 1e9 / (ms / 1e3), 1)}
-    stages["device_total_ms"] = round(statistics.mean(per_stage["total"]), 4)
-    scan_ms = stages["bwd"]["ms"] + stages["fwd_post"]["ms"]
-    scan_gbs = (need["bwd"] + need["fwd_post"]) / 1e9 / (scan_ms / 1e3)
-    stages["scan_plus_posterior"] = {"ms": round(scan_ms, 4), "GBps": round(scan_gbs, 1),
-                                     "frac_of_hbm_peak": round(scan_gbs / HBM_PEAK_GBS, 4)}
-    dominant = max(("bwd", "fwd_post", "beam", "sequence"), key=lambda k: stages[k]["ms"])
-    traffic = MEASURED_TRAFFIC_GB.get((a.workload, N, dominant))
+    for k in ("scan", "bwd", "fwd_post", "beam", "sequence"):
+        if mean[k] > 0:
+            stages[k] = {"ms": round(mean[k], 4), "algorithmic_GB": round(need[k] / 1e9, 4),
+                         "GBps": round(need[k] / 1e9 / (mean[k] / 1e3), 1)}
+    stages["device_total_ms"] = round(mean["total"], 4)
+    stages["scan_plus_posterior"] = scan_stage(need, mean)
+    scan_gbs = stages["scan_plus_posterior"]["GBps"]
+    dominant = max((k for k in ("scan", "bwd", "fwd_post", "beam", "sequence") if k in stages), key=lambda k: stages[k]["ms"])
     roofline = {"bound": "hbm", "kernel": dominant, "achieved": stages[dominant]["GBps"], "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(stages[dominant]["GBps"] / HBM_PEAK_GBS, 4),
-                "traffic": None if traffic is None else round(traffic * 1e9)}
+                "traffic": measured_traffic(a.workload, N, a.columns, dominant)}
 
-    # the same batch with the hardware-exp/log scan arithmetic, for comparison (not `value`)
-    other = None
-    if a.scan_mode != "fast" and a.alt_steps > 0:
-        gpubuf.set_scan_mode("fast")
-        alt = {k: [] for k in api.STAGES}
-        api.openfish_decode_gpu_discard(T, N, C, scores, state_len, opt, gpubuf)
-        t1 = time.perf_counter()
-        for _ in range(a.alt_steps):
-            api.openfish_decode_gpu_discard(T, N, C, scores, state_len, opt, gpubuf)
-            for k, v in gpubuf.timings().items():
-                alt[k].append(v)
-        alt_ms = 1e3 * (time.perf_counter() - t1) / a.alt_steps
+    # side measurements on the same batch (never `value`): the other arrangement of the scans, and the
+    # hardware-exp/log scan arithmetic (not parity-grade)
+    def side(split, mode, note):
+        gpubuf.set_split_scans(split)
+        gpubuf.set_scan_mode(mode)
+        api.openfish_decode_gpu_discard(*call, gpubuf)
+        ms, mn = timed_decodes(api, gpubuf, call, a.alt_steps)
+        gpubuf.set_split_scans(a.split_scans)
         gpubuf.set_scan_mode(a.scan_mode)
-        fb, ff = statistics.mean(alt["bwd"]), statistics.mean(alt["fwd_post"])
-        other = {"chunks_per_s": round(N / (alt_ms / 1e3), 1), "ms_per_step": round(alt_ms, 4),
-                 "bwd_ms": round(fb, 4), "fwd_post_ms": round(ff, 4),
-                 "scan_plus_posterior_GBps": round((need["bwd"] + need["fwd_post"]) / 1e9 / ((fb + ff) / 1e3), 1),
-                 "note": "scans with v_exp_f32/v_log_f32: bwd within 2 ulp, a few posteriors per ten million beyond 1e-3 relative"}
+        return {"chunks_per_s": round(N / (ms / 1e3), 1), "ms_per_step": round(ms, 4),
+                "stage_ms": {k: round(v, 4) for k, v in mn.items() if v > 0},
+                "scan_plus_posterior": scan_stage(need, mn), "note": note}
+
+    other_split, fast_mode = None, None
+    if a.alt_steps > 0:
+        other_split = side(not a.split_scans, a.scan_mode,
+                           "split scans: backward scan, then forward scan + posterior on a second stream beside the beam search"
+                           if not a.split_scans else "both scans and the posterior as one kernel, then the beam search")
+        if a.scan_mode != "fast":
+            fast_mode = side(a.split_scans, "fast",
+                             "scans with v_exp_f32/v_log_f32 only: bwd within 2 ulp, a few posteriors per ten million "
+                             "beyond 1e-3 relative; outside the acceptance bar, shown as the memory-bound floor of the kernels")
 
     # two batches in flight from one thread: enqueue on one gpubuf while the other one's decode
     # runs (the blocking call is enqueue + wait + copies into fresh host buffers)
@@ -228,11 +256,12 @@ def main():
     if a.overlap_steps > 0:
         bufs = [gpubuf, api.GpuBuf(T, N, state_len)]
         bufs[1].set_scan_mode(a.scan_mode)
-        api.openfish_decode_gpu(T, N, C, scores, state_len, opt, bufs[1])
+        bufs[1].set_split_scans(a.split_scans)
+        api.openfish_decode_gpu(*call, bufs[1])
         t2 = time.perf_counter()
-        api.openfish_amd_decode_enqueue(T, N, C, scores, state_len, opt, bufs[0])
+        api.openfish_amd_decode_enqueue(*call, bufs[0])
         for k in range(1, 2 * a.overlap_steps):
-            api.openfish_amd_decode_enqueue(T, N, C, scores, state_len, opt, bufs[k % 2])
+            api.openfish_amd_decode_enqueue(*call, bufs[k % 2])
             api.openfish_amd_decode_wait(bufs[(k - 1) % 2], copy=False)
         api.openfish_amd_decode_wait(bufs[(2 * a.overlap_steps - 1) % 2], copy=False)
         sec = time.perf_counter() - t2
@@ -268,13 +297,14 @@ def main():
         "metric": "CRF chunks decoded/sec at %s (%d states, T=%d, N=%d); achieved HBM GB/s" % (a.workload, S, T, N),
         "value": round(N / (ms_per_step / 1e3), 1), "unit": "chunks/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        # state values and scores are fp32 (fp16 inputs); the default scans evaluate exp/log in fp64
+        # state values and scores are fp32 (fp16 inputs); the default scans evaluate exp/log in fp64 where the
+        # fp32 estimate is not provably the CPU path's result
         "vs_baseline": None, "dtype": "f32" if a.scan_mode == "fast" else "f32+f64", "data": "synthetic",
-        "config": {"workload": "%s: state_len %d, S=%d, C=%d fp16 TNC, T=%d, N=%d, beam 32, beam_cut 100, blank 2.0"
-                               % (a.workload, state_len, S, C, T, N),
-                   "scan_mode": a.scan_mode, "seed": a.seed},
-        "roofline": roofline, "stages": stages, "fast_scan_mode": other, "two_in_flight": overlap,
-        "cpu_baseline": cpu,
+        "config": {"workload": "%s: state_len %d, S=%d, C=%d fp16 TNC (%d columns per state), T=%d, N=%d, beam 32, "
+                               "beam_cut 100, blank 2.0" % (a.workload, state_len, S, C, a.columns, T, N),
+                   "scan_mode": a.scan_mode, "scans": "split" if a.split_scans else "one kernel", "seed": a.seed},
+        "roofline": roofline, "stages": stages, "other_scan_arrangement": other_split, "fast_scan_mode": fast_mode,
+        "two_in_flight": overlap, "cpu_baseline": cpu,
     }))
 
 
