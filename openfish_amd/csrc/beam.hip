@@ -200,21 +200,28 @@ struct Vec<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
 template <>
 struct Vec<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
 
-// one wave's share of a row of ROW_BYTES bytes: lane l owns vectors (i*64 + l)
+// one wave's share of a row of ROW_BYTES bytes: lane l owns vectors (i*64 + l).  Rows of 256
+// and 512 bytes are split into 4- and 8-byte vectors, one per lane; all others into 16-byte
+// vectors, of which the last round may cover only the lower lanes (rows of five-column scores
+// are 640, 2560 or 10240 bytes).
 template <int ROW_BYTES>
 struct RowRegs {
-    static constexpr int kPer = ROW_BYTES / 64;
-    static constexpr int kVec = kPer >= 16 ? 16 : kPer;
-    static constexpr int kCnt = kPer / kVec;
+    static constexpr int kVec = ROW_BYTES == 256 ? 4 : ROW_BYTES == 512 ? 8 : 16;
+    static constexpr int kVecs = ROW_BYTES / kVec;
+    static constexpr int kCnt = (kVecs + 63) / 64;
+    static_assert(ROW_BYTES % kVec == 0, "rows are whole vectors");
     typedef typename Vec<kVec>::type V;
     V v[kCnt];
+    static __device__ __forceinline__ bool mine(int i, int lane) { return (i + 1) * 64 <= kVecs || i * 64 + lane < kVecs; }
     __device__ __forceinline__ void load(const char *row, int lane) {
 #pragma unroll
-        for (int i = 0; i < kCnt; ++i) v[i] = *reinterpret_cast<const V *>(row + (size_t)(i * 64 + lane) * kVec);
+        for (int i = 0; i < kCnt; ++i)
+            if (mine(i, lane)) v[i] = *reinterpret_cast<const V *>(row + (size_t)(i * 64 + lane) * kVec);
     }
     __device__ __forceinline__ void store(char *row, int lane) const {
 #pragma unroll
-        for (int i = 0; i < kCnt; ++i) *reinterpret_cast<V *>(row + (size_t)(i * 64 + lane) * kVec) = v[i];
+        for (int i = 0; i < kCnt; ++i)
+            if (mine(i, lane)) *reinterpret_cast<V *>(row + (size_t)(i * 64 + lane) * kVec) = v[i];
     }
 };
 
@@ -252,10 +259,11 @@ struct BeamShared {
     int consumed;          // rows the search wave is done with
 };
 
-// LDS of one chunk
-template <int S>
+// LDS of one chunk.  Score rows are kept as the caller lays them out: COLS = 4 transitions per
+// state, or 5 with an unused blank first.
+template <int S, int COLS>
 struct BeamRing {
-    _Float16 row_s[BeamCfg<S>::kLdsRows][4 * S];
+    _Float16 row_s[BeamCfg<S>::kLdsRows][COLS * S];
     float row_b[BeamCfg<S>::kLdsRows][S];
 };
 template <int S>
@@ -264,17 +272,17 @@ struct BeamTrace {
     int32_t state[BeamCfg<S>::kTraceBlock];
     uint8_t move[BeamCfg<S>::kTraceBlock];
 };
-template <int S>
+template <int S, int COLS>
 struct __attribute__((aligned(16))) BeamLds {
     // the ring is dead once the last time step has read its row; the traceback stages its blocks there
     union {
-        BeamRing<S> ring;
+        BeamRing<S, COLS> ring;
         BeamTrace<S> trace;
     };
     BeamShared sh;
 };
-static_assert(sizeof(BeamTrace<64>) <= sizeof(BeamRing<64>) && sizeof(BeamTrace<256>) <= sizeof(BeamRing<256>) &&
-                  sizeof(BeamTrace<1024>) <= sizeof(BeamRing<1024>),
+static_assert(sizeof(BeamTrace<64>) <= sizeof(BeamRing<64, 4>) && sizeof(BeamTrace<256>) <= sizeof(BeamRing<256, 4>) &&
+                  sizeof(BeamTrace<1024>) <= sizeof(BeamRing<1024, 4>),
               "traceback staging must fit into the ring");
 
 // CPG chunks per workgroup.  The waves of a group are dealt round over the four SIMDs of
@@ -282,7 +290,7 @@ static_assert(sizeof(BeamTrace<64>) <= sizeof(BeamRing<64>) && sizeof(BeamTrace<
 // to pile onto two SIMDs.  With two chunks a group is four waves, two of them searching;
 // with four chunks it is eight waves and every SIMD holds exactly one search wave and one
 // loader, which is what a batch of more than two chunks per compute unit needs.
-template <int S, int CPG>
+template <int S, int CPG, int COLS>
 __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restrict__ scores,
                                                    const float *__restrict__ bwd,
                                                    ofk_beam_slot_t *__restrict__ beam,
@@ -296,7 +304,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     constexpr int TB = Cfg::kTraceBlock;
 
     constexpr int kGroupChunks = CPG;
-    __shared__ BeamLds<S> lds[kGroupChunks];
+    __shared__ BeamLds<S, COLS> lds[kGroupChunks];
     __shared__ double lse[OFK_LSE_DOUBLES];  // coefficient table of the folds, one copy per workgroup
 
     // waves 0 .. kGroupChunks-1 search, the others load; wave k and wave k + kGroupChunks share a chunk
@@ -310,8 +318,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     auto &trace = lds[member].trace.slot;
     auto &trace_state = lds[member].trace.state;
     auto &trace_move = lds[member].trace.move;
-    const size_t row_stride = (size_t)N * 4 * S;
-    const _Float16 *sc_n = scores + (size_t)n * 4 * S;
+    const size_t row_stride = (size_t)N * COLS * S;
+    const _Float16 *sc_n = scores + (size_t)n * COLS * S;
     const float *bw_n = bwd + (size_t)n * (size_t)(T + 1) * S;
 
     if (wave < kGroupChunks && lane == 0) {
@@ -326,15 +334,15 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // ---- loader wave: row t = (scores[t], bwd[t+1]) into ring slot t % LR ----
         // The ring is spelled out as named registers (not an array indexed by a loop that
         // also contains the spin wait) so that every row stays in VGPRs.
-        RowRegs<8 * S> s0, s1, s2, s3, s4, s5;
+        RowRegs<2 * COLS * S> s0, s1, s2, s3, s4, s5;
         RowRegs<4 * S> g0, g1, g2, g3, g4, g5;
-        auto fetch = [&](RowRegs<8 * S> &rs, RowRegs<4 * S> &rb, int t) {
+        auto fetch = [&](RowRegs<2 * COLS * S> &rs, RowRegs<4 * S> &rb, int t) {
             if (t < T) {
                 rs.load(reinterpret_cast<const char *>(sc_n + (size_t)t * row_stride), lane);
                 rb.load(reinterpret_cast<const char *>(bw_n + (size_t)(t + 1) * S), lane);
             }
         };
-        auto hand_over = [&](RowRegs<8 * S> &rs, RowRegs<4 * S> &rb, int t) {
+        auto hand_over = [&](RowRegs<2 * COLS * S> &rs, RowRegs<4 * S> &rb, int t) {
             if (t < T) {
                 // the ring is full most of the time (a search step takes about 3000 cycles): poll
                 // seldom, the rows in registers and in the ring leave ample slack for waking up late
@@ -449,8 +457,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         const float *rb = row_b[slot];
         const int lo4 = (state << 2) & (S - 1);
         const int top = state >> (BITS - 2);
-        r0h = rs[4 * (lo4 + b0) + top];
-        r1h = rs[4 * (lo4 + b0 + 1) + top];
+        r0h = rs[COLS * (lo4 + b0) + (COLS - 4) + top];
+        r1h = rs[COLS * (lo4 + b0 + 1) + (COLS - 4) + top];
         g01 = *reinterpret_cast<const float2 *>(&rb[lo4 + b0]);
         gst = rb[state];
         const uint4 *hp = reinterpret_cast<const uint4 *>(&sh.hash[16 * h]);
@@ -730,7 +738,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     }
 }
 
-template <int S>
+template <int S, int COLS>
 int launch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
                 uint8_t *moves, int T, int N, float log_cut, float stay, int flags, const double *lse_table,
                 hipStream_t st) {
@@ -738,16 +746,30 @@ int launch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int
     // where the LDS of four chunks fits (64 and 256 states)
     if constexpr (S <= 256) {
         if (N > 512) {
-            hipLaunchKernelGGL((beam_kernel<S, 4>), dim3((N + 3) / 4), dim3(512), 0, st,
+            hipLaunchKernelGGL((beam_kernel<S, 4, COLS>), dim3((N + 3) / 4), dim3(512), 0, st,
                                static_cast<const _Float16 *>(scores), bwd, beam, states, moves, T, N, log_cut,
                                stay, flags, lse_table);
             return (int)hipGetLastError();
         }
     }
-    hipLaunchKernelGGL((beam_kernel<S, 2>), dim3((N + 1) / 2), dim3(256), 0, st,
+    hipLaunchKernelGGL((beam_kernel<S, 2, COLS>), dim3((N + 1) / 2), dim3(256), 0, st,
                            static_cast<const _Float16 *>(scores), bwd, beam, states, moves, T, N, log_cut, stay,
                            flags, lse_table);
     return (int)hipGetLastError();
+}
+
+int dispatch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states, uint8_t *moves,
+                  int T, int N, int state_len, int columns, float log_cut, float stay, int flags,
+                  const double *lse_table, hipStream_t st) {
+    switch (state_len * 8 + columns) {
+        case 3 * 8 + 4: return launch_beam<64, 4>(scores, bwd, beam, states, moves, T, N, log_cut, stay, flags, lse_table, st);
+        case 4 * 8 + 4: return launch_beam<256, 4>(scores, bwd, beam, states, moves, T, N, log_cut, stay, flags, lse_table, st);
+        case 5 * 8 + 4: return launch_beam<1024, 4>(scores, bwd, beam, states, moves, T, N, log_cut, stay, flags, lse_table, st);
+        case 3 * 8 + 5: return launch_beam<64, 5>(scores, bwd, beam, states, moves, T, N, log_cut, stay, flags, lse_table, st);
+        case 4 * 8 + 5: return launch_beam<256, 5>(scores, bwd, beam, states, moves, T, N, log_cut, stay, flags, lse_table, st);
+        case 5 * 8 + 5: return launch_beam<1024, 5>(scores, bwd, beam, states, moves, T, N, log_cut, stay, flags, lse_table, st);
+        default: return OFK_BAD_ARGS;
+    }
 }
 
 }  // namespace
@@ -771,7 +793,7 @@ std::mutex g_scratch_mutex;
 }  // namespace
 
 extern "C" int ofk_beam_search_static(const void *scores, const float *bwd, int32_t *states, uint8_t *moves, int T,
-                                      int N, int state_len, float log_beam_cut, float stay,
+                                      int N, int state_len, int columns, float log_beam_cut, float stay,
                                       const double *lse_table_host, int flags, void *stream) {
     if (!scores || !bwd || !states || !moves || !lse_table_host || T < 1 || N < 1) return OFK_BAD_ARGS;
     if ((reinterpret_cast<uintptr_t>(scores) | reinterpret_cast<uintptr_t>(bwd)) & 15u) return OFK_BAD_ARGS;
@@ -798,25 +820,17 @@ extern "C" int ofk_beam_search_static(const void *scores, const float *bwd, int3
     ofk_beam_slot_t *beam = reinterpret_cast<ofk_beam_slot_t *>(base + kStaticTableBytes);
     const double *lse_table = reinterpret_cast<const double *>(base);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    switch (state_len) {
-        case 3: return launch_beam<64>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
-        case 4: return launch_beam<256>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
-        case 5: return launch_beam<1024>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
-        default: return OFK_BAD_ARGS;
-    }
+    return dispatch_beam(scores, bwd, beam, states, moves, T, N, state_len, columns, log_beam_cut, stay, flags,
+                         lse_table, st);
 }
 
 extern "C" int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
-                               uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
-                               const double *lse_table, int flags, void *stream) {
+                               uint8_t *moves, int T, int N, int state_len, int columns, float log_beam_cut,
+                               float stay, const double *lse_table, int flags, void *stream) {
     if (!scores || !bwd || !beam || !states || !moves || !lse_table || T < 1 || N < 1) return OFK_BAD_ARGS;
     if ((reinterpret_cast<uintptr_t>(scores) | reinterpret_cast<uintptr_t>(bwd) | reinterpret_cast<uintptr_t>(beam)) & 15u)
         return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    switch (state_len) {
-        case 3: return launch_beam<64>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
-        case 4: return launch_beam<256>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
-        case 5: return launch_beam<1024>(scores, bwd, beam, states, moves, T, N, log_beam_cut, stay, flags, lse_table, st);
-        default: return OFK_BAD_ARGS;
-    }
+    return dispatch_beam(scores, bwd, beam, states, moves, T, N, state_len, columns, log_beam_cut, stay, flags,
+                         lse_table, st);
 }

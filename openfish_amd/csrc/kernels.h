@@ -28,20 +28,22 @@ typedef uint16_t ofk_beam_slot_t;
  *                      as OFK_SCAN_PRECISE);
  *   OFK_SCAN_PRECISE   the CPU path's double exp/log and fp32 roundings everywhere;
  *   OFK_SCAN_FAST      hardware fp32 exp/log everywhere (last-bit differences).
- * spl: states per lane, 4, 2 or 1; 0 chooses from the batch size. */
+ * spl: states per lane, 4, 2 or 1; 0 chooses from the batch size.
+ * columns: fp16 values per state in scores, 4 (the transitions) or 5 (an unused blank, then the
+ * transitions); five-column scores are read where they lie. */
 #define OFK_SCAN_TWO_TIER 0
 #define OFK_SCAN_PRECISE 1
 #define OFK_SCAN_FAST 2
-int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, float stay, int mode,
+int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, int columns, float stay, int mode,
                  int spl, void *stream);
-int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N,
-                      int state_len, float stay, int mode, int spl, void *stream);
+int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N, int state_len,
+                      int columns, float stay, int mode, int spl, void *stream);
 /* Both sweeps and the posterior in one kernel: the forward and backward recursions of a chunk run
  * side by side in one workgroup and meet in the middle of the chunk (same tensors as
  * ofk_bwd_scan followed by ofk_fwd_post_scan).  Rows 0 .. T/2-1 of post hold forward values
  * while the kernel runs. */
 int ofk_scan_posterior(const void *scores, float *bwd, float *post, int T, int N, int state_len,
-                       float stay, int mode, int spl, void *stream);
+                       int columns, float stay, int mode, int spl, void *stream);
 /* Table behind log(1 + e^-gap), the correction of a pairwise log-sum-exp, for gap in
  * [0, 17): OFK_LSE_CELLS cells of width 1/4, each a degree-8 polynomial in
  * s = 8 * (gap - centre) in [-1, 1], coefficients lowest degree first.  Built on the
@@ -51,7 +53,7 @@ int ofk_scan_posterior(const void *scores, float *bwd, float *post, int T, int N
 #define OFK_LSE_DOUBLES (OFK_LSE_CELLS * OFK_LSE_COEFS)
 
 int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int32_t *states,
-                    uint8_t *moves, int T, int N, int state_len, float log_beam_cut, float stay,
+                    uint8_t *moves, int T, int N, int state_len, int columns, float log_beam_cut, float stay,
                     const double *lse_table, int flags, void *stream);
 /* The same search with the beam slots and the table in a static device array of the library
  * (OFK_STATIC_SLOT_BYTES of slots: N * (T + 1) * 64 bytes must fit, else OFK_TOO_LARGE and nothing
@@ -60,8 +62,8 @@ int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam,
  * one device share the array and race. */
 #define OFK_STATIC_SLOT_BYTES (64u << 20)
 int ofk_beam_search_static(const void *scores, const float *bwd, int32_t *states, uint8_t *moves, int T, int N,
-                           int state_len, float log_beam_cut, float stay, const double *lse_table_host, int flags,
-                           void *stream);
+                           int state_len, int columns, float log_beam_cut, float stay, const double *lse_table_host,
+                           int flags, void *stream);
 /* flags bit 0: replay every stay/step merge one by one in CPU order (the path otherwise taken
  * only after a hash collision); results must not change.  For tests. */
 /* Phred characters run from '"' (34, q = 1) to 'S' (83, q = 50).  thr[j] is the smallest
@@ -77,9 +79,6 @@ int ofk_sequence(const float *post, int32_t *states, const uint8_t *moves, float
                  int state_len, const ofk_phred_table_t *phred, void *stream);
 /* device-to-device copy of `bytes` (a multiple of 16); the calibration kernel for counters */
 int ofk_copy(void *dst, const void *src, size_t bytes, void *stream);
-/* fp16 [groups][5] -> [groups][4], dropping element 0 of every group (the blank column of a
- * five-column CRF head); groups = T * N * S */
-int ofk_drop_blank_column(const void *scores5, void *scores4, size_t groups, void *stream);
 int ofk_rotary_emb(void *x, const float *sin_buf, const float *cos_buf, int batch, int seqlen,
                    int nheads, int rotary_half, long stride_batch, long stride_seq, long stride_head,
                    void *stream);

@@ -126,8 +126,6 @@ typedef struct {
     void *slab;            /* one device allocation behind all pub fields */
     unsigned char *h_out;  /* pinned staging for moves | sequence | qstring */
     double *lse_table;     /* device copy of the log(1 + e^-gap) table */
-    void *scores4;         /* four-column copy of a five-column score tensor, allocated on first use */
-    size_t scores4_bytes;
     hipStream_t s_main, s_side;
     hipEvent_t ev[EV_COUNT];
     float ms[OPENFISH_AMD_STAGE_COUNT];
@@ -208,7 +206,6 @@ void openfish_gpubuf_free(openfish_gpubuf_t *gpubuf) {
     HIP_OK(hipStreamDestroy(g->s_side));
     HIP_OK(hipHostFree(g->h_out));
     HIP_OK(hipFree(g->lse_table));
-    if (g->scores4) HIP_OK(hipFree(g->scores4));
     HIP_OK(hipFree(g->slab));
     g->magic = 0;
     free(g);
@@ -224,40 +221,22 @@ static ofa_gpubuf_t *checked(const openfish_gpubuf_t *gpubuf, int T, int N, int 
     return g;
 }
 
-static void check_scores_any(int T, int N, int C, const void *scores, int state_len, const openfish_opt_t *opt,
-                             int allow_blank_column) {
+/* Scores carry, per state, the four step columns, or five with a blank/stay column first (as a
+ * CRF head emits them before the blank is dropped).  The kernels read either layout where it
+ * lies and never look at the blank column: the stay score is options->blank_score, as for any
+ * other input (reference src/beam_search.c:213). */
+static void check_scores(int T, int N, int C, const void *scores, int state_len, const openfish_opt_t *opt) {
     check_state_len(state_len);
     if (T < 1 || N < 1) die("T and N must be positive");
     if (T > OFK_MAX_T) die("chunks longer than 8192 time steps are not supported");
-    if (C != 4 * states_of(state_len) && !(allow_blank_column && C == 5 * states_of(state_len)))
-        die(allow_blank_column
-                ? "C must be 4 * 4^state_len (one score per state and dropped base) or 5 * 4^state_len (a blank "
-                  "column first)"
-                : "C must be 4 * 4^state_len (one score per state and dropped base)");
+    if (C != 4 * states_of(state_len) && C != 5 * states_of(state_len))
+        die("C must be 4 * 4^state_len (one score per state and dropped base) or 5 * 4^state_len (a blank "
+            "column first)");
     if (!scores) die("scores_TNC is NULL");
     if (!opt) die("options is NULL");
 }
 
-static void check_scores(int T, int N, int C, const void *scores, int state_len, const openfish_opt_t *opt) {
-    check_scores_any(T, N, C, scores, state_len, opt, 0);
-}
-
-/* A five-column tensor (C = 5 * 4^state_len: a blank/stay column, then the four step columns
- * of every state, as a CRF head emits them before the blank is dropped) is reduced to the
- * four-column layout the decoder consumes; the stay score is options->blank_score, as for
- * any other input (reference src/beam_search.c:213). */
-static const void *four_columns(ofa_gpubuf_t *g, int T, int N, int C, const void *scores, int state_len) {
-    const size_t S = (size_t)states_of(state_len);
-    if ((size_t)C == 4 * S) return scores;
-    const size_t groups = (size_t)T * (size_t)N * S, bytes = groups * 8;
-    if (g->scores4_bytes < bytes) {
-        if (g->scores4) HIP_OK(hipFree(g->scores4));
-        HIP_OK(hipMalloc(&g->scores4, bytes));
-        g->scores4_bytes = bytes;
-    }
-    launch_ok(ofk_drop_blank_column(scores, g->scores4, groups, g->s_main), "drop_blank_column");
-    return g->scores4;
-}
+static int columns_of(int C, int state_len) { return C / states_of(state_len); }
 
 static float log_beam_cut(const openfish_opt_t *opt) {
     /* reference src/beam_search.c:135 */
@@ -374,28 +353,28 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
 
     join_null_stream(g);
     HIP_OK(hipEventRecord(g->ev[EV_START], g->s_main));
-    scores_TNC = four_columns(g, T, N, C, scores_TNC, state_len);
+    const int cols = columns_of(C, state_len);
     /* The one-kernel scans walk every chunk from both ends at once; when a time step of the score
      * tensor is a multiple of 4 MiB apart from the next (2048 chunks of 256 states, 512 of 1024),
      * those streams all land on the same memory channels and the kernel runs at half its speed
      * (measured 9.9 ms against 6.2 ms for the split scans at 2048 x 256): the split scans take over. */
-    const size_t step_bytes = (size_t)N * 4 * (size_t)states_of(state_len) * 2;
+    const size_t step_bytes = (size_t)N * (size_t)C * 2;
     g->pend_split = g->split_scans || step_bytes % ((size_t)4 << 20) == 0;
     if (!g->pend_split) {
         /* both sweeps and the posterior in one kernel, then the beam search, all on one stream */
-        launch_ok(ofk_scan_posterior(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->scan_mode,
+        launch_ok(ofk_scan_posterior(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, cols, stay, g->scan_mode,
                                      g->scan_spl, g->s_main), "scan_posterior");
         HIP_OK(hipEventRecord(g->ev[EV_BWD_END], g->s_main));
         HIP_OK(hipEventRecord(g->ev[EV_BEAM_START], g->s_main));
         launch_ok(ofk_beam_search(scores_TNC, g->pub.bwd_NTC, (ofk_beam_slot_t *)g->pub.beam_vector,
-                                  (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, log_beam_cut(options),
+                                  (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, cols, log_beam_cut(options),
                                   stay, g->lse_table, g->debug_flags, g->s_main), "beam_search");
         HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_main));
         /* the moves are final once the beam search is: they travel while the sequence stage runs */
         HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BEAM_END], 0));
         HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_side));
     } else {
-        launch_ok(ofk_bwd_scan(scores_TNC, g->pub.bwd_NTC, T, N, state_len, stay, g->scan_mode, g->scan_spl, g->s_main),
+        launch_ok(ofk_bwd_scan(scores_TNC, g->pub.bwd_NTC, T, N, state_len, cols, stay, g->scan_mode, g->scan_spl, g->s_main),
                   "bwd_scan");
         HIP_OK(hipEventRecord(g->ev[EV_BWD_END], g->s_main));
 
@@ -404,12 +383,12 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
          * the backward sweep ran on and so starts first; the forward sweep follows through an event. */
         HIP_OK(hipEventRecord(g->ev[EV_BEAM_START], g->s_main));
         launch_ok(ofk_beam_search(scores_TNC, g->pub.bwd_NTC, (ofk_beam_slot_t *)g->pub.beam_vector,
-                                  (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, log_beam_cut(options),
+                                  (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, cols, log_beam_cut(options),
                                   stay, g->lse_table, g->debug_flags, g->s_main), "beam_search");
         HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_main));
 
         HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BWD_END], 0));
-        launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, stay, g->scan_mode,
+        launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, cols, stay, g->scan_mode,
                                     g->scan_spl, g->s_side), "fwd_post_scan");
         HIP_OK(hipEventRecord(g->ev[EV_FWD_END], g->s_side));
         /* the moves are final once the beam search is: they travel while the sequence stage runs */
@@ -433,7 +412,7 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
 void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC, const int state_len,
                          const openfish_opt_t *options, const openfish_gpubuf_t *gpubuf, uint8_t **moves,
                          char **sequence, char **qstring) {
-    check_scores_any(T, N, C, scores_TNC, state_len, options, 1);
+    check_scores(T, N, C, scores_TNC, state_len, options);
     if (!moves || !sequence || !qstring) die("decode: output pointer is NULL");
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     const size_t nt = (size_t)N * (size_t)T;
@@ -452,7 +431,7 @@ void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC
 
 void openfish_amd_decode_enqueue(int T, int N, int C, const void *scores_TNC, int state_len,
                                  const openfish_opt_t *options, const openfish_gpubuf_t *gpubuf) {
-    check_scores_any(T, N, C, scores_TNC, state_len, options, 1);
+    check_scores(T, N, C, scores_TNC, state_len, options);
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     enqueue_decode(g, T, N, C, scores_TNC, state_len, options);
 }
@@ -505,7 +484,7 @@ void openfish_amd_bwd_scan(int T, int N, int C, const void *scores, int state_le
     openfish_opt_t o = DECODER_INIT;
     check_scores(T, N, C, scores, state_len, &o);
     check_scan_mode(scan_mode);
-    launch_ok(ofk_bwd_scan(scores, bwd, T, N, state_len, stay_score, scan_mode, 0, NULL), "bwd_scan");
+    launch_ok(ofk_bwd_scan(scores, bwd, T, N, state_len, columns_of(C, state_len), stay_score, scan_mode, 0, NULL), "bwd_scan");
     HIP_OK(hipStreamSynchronize(0));
 }
 
@@ -514,7 +493,7 @@ void openfish_amd_fwd_post_scan(int T, int N, int C, const void *scores, int sta
     openfish_opt_t o = DECODER_INIT;
     check_scores(T, N, C, scores, state_len, &o);
     check_scan_mode(scan_mode);
-    launch_ok(ofk_fwd_post_scan(scores, bwd, post, T, N, state_len, stay_score, scan_mode, 0, NULL), "fwd_post_scan");
+    launch_ok(ofk_fwd_post_scan(scores, bwd, post, T, N, state_len, columns_of(C, state_len), stay_score, scan_mode, 0, NULL), "fwd_post_scan");
     HIP_OK(hipStreamSynchronize(0));
 }
 
@@ -523,7 +502,7 @@ void openfish_amd_scan_posterior(int T, int N, int C, const void *scores, int st
     openfish_opt_t o = DECODER_INIT;
     check_scores(T, N, C, scores, state_len, &o);
     check_scan_mode(scan_mode);
-    launch_ok(ofk_scan_posterior(scores, bwd, post, T, N, state_len, stay_score, scan_mode, 0, NULL), "scan_posterior");
+    launch_ok(ofk_scan_posterior(scores, bwd, post, T, N, state_len, columns_of(C, state_len), stay_score, scan_mode, 0, NULL), "scan_posterior");
     HIP_OK(hipStreamSynchronize(0));
 }
 
@@ -532,7 +511,8 @@ void openfish_amd_beam_search(int T, int N, int C, const void *scores, int state
     check_scores(T, N, C, scores, state_len, options);
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     launch_ok(ofk_beam_search(scores, bwd, (ofk_beam_slot_t *)g->pub.beam_vector, (int32_t *)g->pub.states,
-                              g->pub.moves, T, N, state_len, log_beam_cut(options), options->blank_score,
+                              g->pub.moves, T, N, state_len, columns_of(C, state_len), log_beam_cut(options),
+                              options->blank_score,
                               g->lse_table, g->debug_flags, NULL),
               "beam_search");
     HIP_OK(hipStreamSynchronize(0));
@@ -545,7 +525,8 @@ void openfish_amd_beam_search_static(int T, int N, int C, const void *scores, in
     if (!bwd || !states || !moves) die("beam_search_static: bwd, states and moves must be device pointers");
     double tab[OFK_LSE_DOUBLES]; /* read by the first call on a device only */
     build_lse_table(tab);
-    const int rc = ofk_beam_search_static(scores, bwd, states, moves, T, N, state_len, log_beam_cut(options),
+    const int rc = ofk_beam_search_static(scores, bwd, states, moves, T, N, state_len, columns_of(C, state_len),
+                                          log_beam_cut(options),
                                           options->blank_score, tab, 0, NULL);
     if (rc == OFK_TOO_LARGE) {
         fprintf(stderr, "openfish: beam_search_static: N * (T + 1) * 64 = %zu bytes of beam slots exceed the static "
@@ -576,7 +557,8 @@ void openfish_amd_decode_from_tensors(int T, int N, int C, const void *scores, i
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     join_null_stream(g);
     launch_ok(ofk_beam_search(scores, bwd, (ofk_beam_slot_t *)g->pub.beam_vector, (int32_t *)g->pub.states,
-                              g->pub.moves, T, N, state_len, log_beam_cut(options), options->blank_score,
+                              g->pub.moves, T, N, state_len, columns_of(C, state_len), log_beam_cut(options),
+                              options->blank_score,
                               g->lse_table, g->debug_flags, g->s_main), "beam_search");
     launch_ok(ofk_sequence(post, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data, g->pub.base_probs,
                            g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N, state_len,

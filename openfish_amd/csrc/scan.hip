@@ -40,6 +40,15 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
+// fp16 scores per state and time step: the four transitions, or five with an unused blank first.
+// The file is compiled once for each layout.
+#ifndef OFK_COLS
+#define OFK_COLS 4
+#endif
+constexpr int kCols = OFK_COLS;
+constexpr int kLead = kCols - 4;
+static_assert(kCols == 4 || kCols == 5, "scores have four or five columns");
+
 constexpr float kLog2e = 1.44269504088896340736f;
 constexpr float kLn2 = 0.69314718055994530942f;
 
@@ -244,20 +253,39 @@ __device__ __forceinline__ float add_half(uint32_t word, float x) {
 }
 
 // The scores one lane needs for one time step, as loaded: fp16 pairs in 32-bit words.
-// Backward: transition b of own state i is element 4b + i of the lane's window.
+// A state's scores are kCols consecutive fp16 values: the four transitions, after kLead
+// values that the decoder never reads (the blank column of five-column scores).  With
+// four columns a lane's window is contiguous and is fetched with vector loads; with five
+// it is fetched two bytes at a time, straight from the caller's layout.
+__device__ __forceinline__ uint32_t half_at(const _Float16 *p) { return *reinterpret_cast<const uint16_t *>(p); }
+__device__ __forceinline__ uint32_t half_pair_at(const _Float16 *p) {
+    if constexpr (kCols == 4) return *reinterpret_cast<const uint32_t *>(p);
+    else return half_at(p) | (half_at(p + 1) << 16);
+}
+
+// Backward: transition b of own state i is element kCols * b + i of the lane's window
+// (word (4b + i) / 2 of w once packed).
 template <int SPL>
 struct BwdRow;
 template <>
 struct BwdRow<4> {
-    uint4 v[2];
+    uint32_t w[8];
     __device__ __forceinline__ void load(const _Float16 *p) {
-        v[0] = reinterpret_cast<const uint4 *>(p)[0];
-        v[1] = reinterpret_cast<const uint4 *>(p)[1];
+        if constexpr (kCols == 4) {
+            const uint4 x = reinterpret_cast<const uint4 *>(p)[0], y = reinterpret_cast<const uint4 *>(p)[1];
+            w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w;
+            w[4] = y.x; w[5] = y.y; w[6] = y.z; w[7] = y.w;
+        } else {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                w[2 * b] = half_pair_at(p + kCols * b);
+                w[2 * b + 1] = half_pair_at(p + kCols * b + 2);
+            }
+        }
     }
     template <int B, int I>
     __device__ __forceinline__ float add(float x) const {
         constexpr int e = 4 * B + I;
-        const uint32_t w[8] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w};
         return add_half<e % 2>(w[e / 2], x);
     }
 };
@@ -266,7 +294,7 @@ struct BwdRow<2> {
     uint32_t v[4];
     __device__ __forceinline__ void load(const _Float16 *p) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) v[b] = *reinterpret_cast<const uint32_t *>(p + 4 * b);
+        for (int b = 0; b < 4; ++b) v[b] = half_pair_at(p + kCols * b);
     }
     template <int B, int I>
     __device__ __forceinline__ float add(float x) const { return add_half<I>(v[B], x); }
@@ -276,46 +304,41 @@ struct BwdRow<1> {
     uint32_t v[4];  // one fp16 value each, in the low half
     __device__ __forceinline__ void load(const _Float16 *p) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) v[b] = *reinterpret_cast<const uint16_t *>(p + 4 * b);
+        for (int b = 0; b < 4; ++b) v[b] = half_at(p + kCols * b);
     }
     template <int B, int I>
     __device__ __forceinline__ float add(float x) const { return add_half<0>(v[B], x); }
 };
 
-// Forward: transition b into own state i is element 4i + b of the lane's window.
+// Forward: transition b into own state i is element kCols * i + b of the lane's window
+// (word (4i + b) / 2 of w once packed).
 template <int SPL>
-struct FwdRow;
-template <>
-struct FwdRow<4> {
-    uint4 v[2];
+struct FwdRow {
+    uint32_t w[2 * SPL];
     __device__ __forceinline__ void load(const _Float16 *p) {
-        v[0] = reinterpret_cast<const uint4 *>(p)[0];
-        v[1] = reinterpret_cast<const uint4 *>(p)[1];
+        if constexpr (kCols == 4 && SPL == 4) {
+            const uint4 x = reinterpret_cast<const uint4 *>(p)[0], y = reinterpret_cast<const uint4 *>(p)[1];
+            w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w;
+            w[4] = y.x; w[5] = y.y; w[6] = y.z; w[7] = y.w;
+        } else if constexpr (kCols == 4 && SPL == 2) {
+            const uint4 x = *reinterpret_cast<const uint4 *>(p);
+            w[0] = x.x; w[1] = x.y; w[2] = x.z; w[3] = x.w;
+        } else if constexpr (kCols == 4) {
+            const uint2 x = *reinterpret_cast<const uint2 *>(p);
+            w[0] = x.x; w[1] = x.y;
+        } else {
+#pragma unroll
+            for (int i = 0; i < SPL; ++i) {
+                w[2 * i] = half_pair_at(p + kCols * i);
+                w[2 * i + 1] = half_pair_at(p + kCols * i + 2);
+            }
+        }
     }
     template <int I, int B>
     __device__ __forceinline__ float add(float x) const {
         constexpr int e = 4 * I + B;
-        const uint32_t w[8] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w};
         return add_half<e % 2>(w[e / 2], x);
     }
-};
-template <>
-struct FwdRow<2> {
-    uint4 v;
-    __device__ __forceinline__ void load(const _Float16 *p) { v = *reinterpret_cast<const uint4 *>(p); }
-    template <int I, int B>
-    __device__ __forceinline__ float add(float x) const {
-        constexpr int e = 4 * I + B;
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-        return add_half<e % 2>(w[e / 2], x);
-    }
-};
-template <>
-struct FwdRow<1> {
-    uint2 v;
-    __device__ __forceinline__ void load(const _Float16 *p) { v = *reinterpret_cast<const uint2 *>(p); }
-    template <int I, int B>
-    __device__ __forceinline__ float add(float x) const { return add_half<B % 2>(B / 2 ? v.y : v.x, x); }
 };
 
 // SPL consecutive floats in global or shared memory
@@ -383,8 +406,8 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
     const bool live = n < N;
     if (!live) n = N - 1;
 
-    const size_t row_stride = (size_t)N * 4 * S;  // fp16 elements between time steps
-    const _Float16 *sp = scores + (size_t)n * 4 * S + 16 * r + c0;
+    const size_t row_stride = (size_t)N * kCols * S;  // fp16 elements between time steps
+    const _Float16 *sp = scores + (size_t)n * kCols * S + 4 * kCols * r + kLead + c0;
     float *out = bwd + (size_t)n * (size_t)(T + 1) * S + r + c0 * Q;
 
     float a[SPL];
@@ -454,8 +477,8 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
     const bool live = n < N;
     if (!live) n = N - 1;
 
-    const size_t row_stride = (size_t)N * 4 * S;
-    const _Float16 *sp = scores + (size_t)n * 4 * S + 4 * s0;
+    const size_t row_stride = (size_t)N * kCols * S;
+    const _Float16 *sp = scores + (size_t)n * kCols * S + kCols * s0 + kLead;
     const float *bp = bwd + (size_t)n * (size_t)(T + 1) * S + s0;
     float *pp = post + (size_t)n * (size_t)(T + 1) * S + s0;
 
@@ -631,10 +654,10 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
     const int H = T / 2;  // forward: rows 0..H-1 in phase 1, H..T in phase 2
     // Addresses are a base that is the same for the whole workgroup (kept in scalar registers and
     // stepped from row to row by scalar additions) plus a 32-bit offset of the lane that never changes.
-    const ptrdiff_t row_stride = (ptrdiff_t)N * 4 * S;  // fp16 elements between time steps
+    const ptrdiff_t row_stride = (ptrdiff_t)N * kCols * S;  // fp16 elements between time steps
     const int first_chunk = blockIdx.x * Sh::kChunks;
     const unsigned g_eff = (unsigned)(n - first_chunk);  // chunk within the group (dead lanes repeat the last chunk)
-    const _Float16 *const sc_blk = scores + (size_t)first_chunk * 4 * S;
+    const _Float16 *const sc_blk = scores + (size_t)first_chunk * kCols * S;
     const size_t blk_off = (size_t)first_chunk * (size_t)(T + 1) * S;
     float *const bwd_blk = bwd + blk_off;
     float *const post_blk = post + blk_off;
@@ -643,7 +666,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
     if (!forward) {
         // ------------------------------ backward lanes ------------------------------
         const int r = l / H4, c0 = (l % H4) * SPL;  // own states: r + (c0 + i) * Q
-        const unsigned sc_lane = g_eff * 4 * S + 16 * r + c0;
+        const unsigned sc_lane = g_eff * kCols * S + 4 * kCols * r + kLead + c0;
         const unsigned st_lane = chunk_rows + r + c0 * Q;
         float a[SPL];
 #pragma unroll
@@ -777,7 +800,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
     } else {
         // ------------------------------ forward lanes ------------------------------
         const int s0 = SPL * l, q = s0 >> 2;  // own states s0 .. s0+SPL-1, all in quad q
-        const unsigned sc_lane = g_eff * 4 * S + 4 * s0;
+        const unsigned sc_lane = g_eff * kCols * S + kCols * s0 + kLead;
         const unsigned st_lane = chunk_rows + s0;
         float f[SPL];
 #pragma unroll
@@ -1024,18 +1047,7 @@ static int fused_states_per_lane(int S, int N, int forced) {
     return min_spl;
 }
 
-#ifdef OFK_TIER_STATS
-extern "C" void ofk_tier_stats(unsigned long long *out, int reset) {
-    hipDeviceSynchronize();
-    hipMemcpyFromSymbol(out, HIP_SYMBOL(g_tier_stats), sizeof(unsigned long long) * 4);
-    if (reset) {
-        unsigned long long z[4] = {0, 0, 0, 0};
-        hipMemcpyToSymbol(HIP_SYMBOL(g_tier_stats), z, sizeof z);
-    }
-}
-#endif
-
-#ifdef OFK_TIER_STATS
+#if defined(OFK_TIER_STATS) && OFK_COLS == 4
 extern "C" void ofk_tier_stats(unsigned long long *out, int reset) {
     (void)hipDeviceSynchronize();
     (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_tier_stats), sizeof(unsigned long long) * 4);
@@ -1046,8 +1058,8 @@ extern "C" void ofk_tier_stats(unsigned long long *out, int reset) {
 }
 #endif
 
-extern "C" int ofk_scan_posterior(const void *scores, float *bwd, float *post, int T, int N, int state_len,
-                                  float stay, int mode, int spl, void *stream) {
+static int scan_posterior(const void *scores, float *bwd, float *post, int T, int N, int state_len, float stay,
+                          int mode, int spl, void *stream) {
     if (!scores || !bwd || !post || T < 1 || N < 1 || !aligned16(scores) || !aligned16(bwd) || !aligned16(post))
         return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -1063,19 +1075,61 @@ extern "C" int ofk_scan_posterior(const void *scores, float *bwd, float *post, i
     }
 }
 
-extern "C" int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, float stay, int mode,
-                            int spl, void *stream) {
+static int bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, float stay, int mode, int spl,
+                    void *stream) {
     if (!scores || !bwd || T < 1 || N < 1 || !aligned16(scores) || !aligned16(bwd)) return OFK_BAD_ARGS;
     if (state_len < 3 || state_len > 5) return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     OFK_DISPATCH(true, launch_bwd, mode, scores, bwd, T, N, stay, st)
 }
 
-extern "C" int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N,
-                                 int state_len, float stay, int mode, int spl, void *stream) {
+static int fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N, int state_len,
+                         float stay, int mode, int spl, void *stream) {
     if (!scores || !bwd || !post || T < 1 || N < 1 || !aligned16(scores) || !aligned16(bwd) || !aligned16(post))
         return OFK_BAD_ARGS;
     if (state_len < 3 || state_len > 5) return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     OFK_DISPATCH(false, launch_fwd, mode, scores, bwd, post, T, N, stay, st)
 }
+
+// The build compiles this file twice: with four columns, which also holds the entry points, and
+// with five, whose kernels the entry points reach through the three functions named *_five.
+#if OFK_COLS == 5
+extern "C" int ofk_scan_posterior_five(const void *scores, float *bwd, float *post, int T, int N, int state_len,
+                                       float stay, int mode, int spl, void *stream) {
+    return scan_posterior(scores, bwd, post, T, N, state_len, stay, mode, spl, stream);
+}
+extern "C" int ofk_bwd_scan_five(const void *scores, float *bwd, int T, int N, int state_len, float stay, int mode,
+                                 int spl, void *stream) {
+    return bwd_scan(scores, bwd, T, N, state_len, stay, mode, spl, stream);
+}
+extern "C" int ofk_fwd_post_scan_five(const void *scores, const float *bwd, float *post, int T, int N,
+                                      int state_len, float stay, int mode, int spl, void *stream) {
+    return fwd_post_scan(scores, bwd, post, T, N, state_len, stay, mode, spl, stream);
+}
+#else
+extern "C" int ofk_scan_posterior_five(const void *, float *, float *, int, int, int, float, int, int, void *);
+extern "C" int ofk_bwd_scan_five(const void *, float *, int, int, int, float, int, int, void *);
+extern "C" int ofk_fwd_post_scan_five(const void *, const float *, float *, int, int, int, float, int, int, void *);
+
+extern "C" int ofk_scan_posterior(const void *scores, float *bwd, float *post, int T, int N, int state_len,
+                                  int columns, float stay, int mode, int spl, void *stream) {
+    if (columns == 5) return ofk_scan_posterior_five(scores, bwd, post, T, N, state_len, stay, mode, spl, stream);
+    if (columns != 4) return OFK_BAD_ARGS;
+    return scan_posterior(scores, bwd, post, T, N, state_len, stay, mode, spl, stream);
+}
+
+extern "C" int ofk_bwd_scan(const void *scores, float *bwd, int T, int N, int state_len, int columns, float stay,
+                            int mode, int spl, void *stream) {
+    if (columns == 5) return ofk_bwd_scan_five(scores, bwd, T, N, state_len, stay, mode, spl, stream);
+    if (columns != 4) return OFK_BAD_ARGS;
+    return bwd_scan(scores, bwd, T, N, state_len, stay, mode, spl, stream);
+}
+
+extern "C" int ofk_fwd_post_scan(const void *scores, const float *bwd, float *post, int T, int N, int state_len,
+                                 int columns, float stay, int mode, int spl, void *stream) {
+    if (columns == 5) return ofk_fwd_post_scan_five(scores, bwd, post, T, N, state_len, stay, mode, spl, stream);
+    if (columns != 4) return OFK_BAD_ARGS;
+    return fwd_post_scan(scores, bwd, post, T, N, state_len, stay, mode, spl, stream);
+}
+#endif

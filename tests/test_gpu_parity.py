@@ -314,18 +314,38 @@ def test_enqueue_and_wait_with_two_batches_in_flight(api):
         del dev
 
 
-@pytest.mark.parametrize("state_len,T,N", [(3, 150, 5), (4, 90, 3), (5, 40, 2)])
+@pytest.mark.parametrize("state_len,T,N", [(3, 150, 5), (4, 90, 3), (5, 40, 2), (4, 333, 40), (3, 64, 9)])
 def test_five_column_input_equals_its_four_column_view(api, state_len, T, N):
-    """C = 5*S: a blank column in front of the four step columns of every state"""
+    """C = 5*S: a blank column in front of the four step columns of every state, read where it
+    lies by every kernel that takes scores; the blank values (poisoned here) are never looked at"""
     S = 4 ** state_len
     four, five = synth.crf_scores(T, N, state_len, seed=55, five_columns=True)
     assert np.array_equal(five.reshape(T, N, S, 5)[..., 1:].reshape(T, N, 4 * S), four)
+    five = five.copy()
+    five.reshape(T, N, S, 5)[..., 0] = np.float16(np.nan)
     kw = dict(q_scale=0.95, q_shift=-0.2)
     ref = O.decode(four.astype(np.float32), state_len, kw, nthreads=4)
     gb = api.GpuBuf(T, N, state_len)
     sc5 = api.upload_scores_to_hip(five)
-    mv, sq, qs = api.openfish_decode_gpu(T, N, 5 * S, sc5, state_len, api.DECODER_INIT(**kw), gb)
-    assert np.array_equal(gb.tensor("bwd_NTC"), ref["bwd"])
+    for split in (False, True):
+        gb.set_split_scans(split)
+        mv, sq, qs = api.openfish_decode_gpu(T, N, 5 * S, sc5, state_len, api.DECODER_INIT(**kw), gb)
+        assert np.array_equal(gb.tensor("bwd_NTC"), ref["bwd"])
+        close(gb.tensor("post_NTC"), ref["post"], POST_ATOL)
+        assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"])
+        assert np.array_equal(qs, ref["qstring"])
+    # the stages one by one, every scan mode
+    for mode in ("two_tier", "precise", "fast"):
+        for scans in (gpu_scans, gpu_scan_posterior):
+            bwd, post = scans(api, five, state_len, mode=mode)
+            if mode == "fast":
+                np.testing.assert_allclose(bwd, ref["bwd"], rtol=3e-7, atol=1e-6)
+            else:
+                assert np.array_equal(bwd, ref["bwd"])
+                close(post, ref["post"], POST_ATOL)
+    (mv, sq, qs), _ = gpu_from_tensors(api, five, state_len, kw, ref["bwd"], ref["post"])
+    assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
+    (mv, sq, qs), _ = gpu_from_tensors(api, five, state_len, kw, ref["bwd"], ref["post"], debug_flags=1)
     assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
 
 
@@ -342,21 +362,25 @@ def test_constant_scores_closed_form(api):
 
 # ---- full benchmark sizes: every chunk against the oracle, plus size-independent properties ----
 
-FULL = [("fast", 3, 1666, 512, False), ("hac", 4, 1666, 512, False),
-        ("sup", 5, 1666, 256, False), ("hac_stress", 4, 1666, 1024, True)]
+FULL = [("fast", 3, 1666, 512, False, 4), ("hac", 4, 1666, 512, False, 4),
+        ("sup", 5, 1666, 256, False, 4), ("hac_stress", 4, 1666, 1024, True, 4),
+        ("fast_five_columns", 3, 1666, 512, False, 5), ("hac_five_columns", 4, 1666, 512, False, 5),
+        ("sup_five_columns", 5, 1666, 256, False, 5)]
 
 
-@pytest.mark.parametrize("name,state_len,T,N,stress", FULL)
-def test_full_size_configurations(api, name, state_len, T, N, stress):
-    """the four benchmark configurations at full size, all N chunks: bwd bit-identical to the
+@pytest.mark.parametrize("name,state_len,T,N,stress,columns", FULL)
+def test_full_size_configurations(api, name, state_len, T, N, stress, columns):
+    """the benchmark configurations at full size (scores with four columns per state, and with
+    the five the network emits), all N chunks: bwd bit-identical to the
     oracle, every posterior within 1e-3 relative, whole-decode moves and sequence identical and
     the phred string within its bound; then the beam/sequence stage fed the oracle's tensors,
     identical bytes for all N chunks"""
-    S, C = 4 ** state_len, 4 * 4 ** state_len
+    S, C = 4 ** state_len, columns * 4 ** state_len
     scale = synth.stress_scale(N) if stress else None
-    s16 = synth.crf_scores(T, N, state_len, seed=2025, chunk_scale=scale, threads=16)
+    made = synth.crf_scores(T, N, state_len, seed=2025, chunk_scale=scale, threads=16, five_columns=columns == 5)
+    s16, given = (made[0], made[1]) if columns == 5 else (made, made)  # s16: what the oracle decodes
     kw = dict(q_scale=0.95, q_shift=-0.2)
-    sc = api.upload_scores_to_hip(s16)
+    sc = api.upload_scores_to_hip(given)
     gb = api.GpuBuf(T, N, state_len)
     mv, sq, qs = api.openfish_decode_gpu(T, N, C, sc, state_len, api.DECODER_INIT(**kw), gb)
 
@@ -389,7 +413,7 @@ def test_full_size_configurations(api, name, state_len, T, N, stress):
     qstring_close(qs1, ref["qstring"], mv)
 
     # beam search + sequence stage on the oracle's own tensors: identical bytes, every chunk
-    (mv2, sq2, qs2), _ = gpu_from_tensors(api, s16, state_len, kw, ref["bwd"], ref["post"])
+    (mv2, sq2, qs2), _ = gpu_from_tensors(api, given, state_len, kw, ref["bwd"], ref["post"])
     assert np.array_equal(mv2, ref["moves"]) and np.array_equal(sq2, ref["sequence"]) and np.array_equal(qs2, ref["qstring"])
 
 

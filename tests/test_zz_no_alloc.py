@@ -17,10 +17,12 @@ def api():
     return _api
 
 
-def both_entry_points(api, state_len, T, N, seed, scale=None, **opt_kw):
+def both_entry_points(api, state_len, T, N, seed, scale=None, columns=4, **opt_kw):
     S = 4 ** state_len
-    C = 4 * S
-    s16 = synth.crf_scores(T, N, state_len, seed=seed, chunk_scale=scale)
+    C = columns * S
+    s16 = synth.crf_scores(T, N, state_len, seed=seed, chunk_scale=scale, five_columns=columns == 5)
+    if columns == 5:
+        s16 = s16[1]
     sc = api.upload_scores_to_hip(s16)
     bwd = api.DeviceBuffer(4 * N * (T + 1) * S)
     api.openfish_amd_bwd_scan(T, N, C, sc, state_len, 2.0, bwd)
@@ -45,3 +47,4 @@ def test_static_scratch_entry_point_matches_the_gpubuf_one_twice(api):
     both_entry_points(api, 4, 150, 3, seed=72)  # smaller: the array still holds the first call's slots
     both_entry_points(api, 3, 90, 5, seed=73, beam_cut=3.0)
     both_entry_points(api, 5, 60, 2, seed=74)
+    both_entry_points(api, 4, 120, 4, seed=75, columns=5)  # scores with a blank column, read in place
