@@ -186,7 +186,10 @@ int openfish_amd_last_timings(const openfish_gpubuf_t *gpubuf, float *ms, int n)
  *   the device a wavefront for the batch at hand.  Results do not depend on it.
  * debug flags: bit 0 makes the beam search replay every stay/step merge serially in the CPU
  *   path's order, the route it otherwise takes only after a CRC collision between beam hashes;
- *   outputs must be identical with and without it.
+ *   outputs must be identical with and without it.  Bit 1 seeds the beam with hashes of
+ *   (state & 15) instead of the state, so that different sequences share hashes and that route
+ *   is found by the search's own duplicate detection; for tests against a CPU search seeded
+ *   the same way, never for real decoding.
  * split scans: 0 (default) runs both scans and the posterior as one kernel, then the beam
  *   search; 1 runs the backward scan, then the forward scan + posterior on a second stream
  *   beside the beam search.  Same results.

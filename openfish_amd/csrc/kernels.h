@@ -64,8 +64,10 @@ int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam,
 int ofk_beam_search_static(const void *scores, const float *bwd, int32_t *states, uint8_t *moves, int T, int N,
                            int state_len, int columns, float log_beam_cut, float stay, const double *lse_table_host,
                            int flags, void *stream);
-/* flags bit 0: replay every stay/step merge one by one in CPU order (the path otherwise taken
- * only after a hash collision); results must not change.  For tests. */
+/* flags, for tests.  Bit 0: replay every stay/step merge one by one in CPU order (the path
+ * otherwise taken only after a hash collision); results must not change.  Bit 1: seed hashes are
+ * taken from (state & 15), so that different sequences share hashes and the search has to notice
+ * the duplicates by itself; results then equal those of a CPU search seeded the same way. */
 /* Phred characters run from '"' (34, q = 1) to 'S' (83, q = 50).  thr[j] is the smallest
  * miss probability x whose character is at most 82 - j (2.0f if no x in [0,1] reaches it),
  * so that char(x) = 83 - #{j : x >= thr[j]}. */

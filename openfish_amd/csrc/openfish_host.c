@@ -135,7 +135,7 @@ typedef struct {
     int pend_split;        /* how its scans were queued (which events were recorded) */
     int scan_mode;         /* OFK_SCAN_*: arithmetic of the scans of this gpubuf's decodes */
     int scan_spl;          /* states per lane of the scans, 0 = chosen from the batch size */
-    int debug_flags;       /* bit 0: serial replay of the beam search's merges */
+    int debug_flags;       /* bit 0: serial replay of the beam search's merges; bit 1: colliding seed hashes */
     int split_scans;       /* 1: backward sweep, then forward sweep beside the beam search; 0: both sweeps in one kernel */
     ofk_phred_table_t phred; /* thresholds for (phred_shift, phred_scale) */
     float phred_shift, phred_scale;
@@ -663,7 +663,7 @@ static ofa_gpubuf_t *owned(const openfish_gpubuf_t *gpubuf) {
 }
 
 void openfish_amd_gpubuf_set_debug_flags(const openfish_gpubuf_t *gpubuf, int flags) {
-    owned(gpubuf)->debug_flags = flags & 1;
+    owned(gpubuf)->debug_flags = flags & 3;
 }
 
 void openfish_amd_gpubuf_set_scan_mode(const openfish_gpubuf_t *gpubuf, int scan_mode) {

@@ -170,6 +170,13 @@ static size_t count_at_least(const float *v, size_t n, float thr) {
     return c;
 }
 
+/* Test knob, not part of the algorithm: seed hashes are taken from (state & mask), so that with a
+ * narrow mask different sequences share hashes from the first block on and the duplicate-hash
+ * branches of the merge loop (several equal hashes, a step matched by two stays) are exercised.
+ * The default mask keeps every bit, which is the reference's seeding (src/beam_search.c:151-175). */
+static uint32_t g_seed_state_mask = 0xFFFFFFFFu;
+void ofo_set_seed_state_mask(uint32_t mask) { g_seed_state_mask = mask; }
+
 void ofo_beam_search(const float *scores, size_t row_stride, const float *bwd, const float *post,
                      int state_bits, size_t T, float beam_cut, float stay_score,
                      int32_t *states, uint8_t *moves, float *qual_data,
@@ -195,7 +202,7 @@ void ofo_beam_search(const float *scores, size_t row_stride, const float *bwd, c
         size_t slot = 0;
         for (size_t s = 0; s < S && slot < W; ++s) {
             if (bwd[s] >= seed_thr) {
-                front[slot].hash = ofo_crc32c(CRC_SEED, (uint32_t)s, 32);
+                front[slot].hash = ofo_crc32c(CRC_SEED, (uint32_t)s & g_seed_state_mask, 32);
                 front[slot].state = (int32_t)s;
                 front[slot].prev = 0;
                 front[slot].stay = 0;

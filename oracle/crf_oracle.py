@@ -53,6 +53,8 @@ def lib():
         L = C.CDLL(ORACLE_SO)
         L.ofo_crc32c.restype = C.c_uint32
         L.ofo_crc32c.argtypes = [C.c_uint32, C.c_uint32, C.c_int]
+        L.ofo_set_seed_state_mask.restype = None
+        L.ofo_set_seed_state_mask.argtypes = [C.c_uint32]
         L.ofo_kth_largest.restype = C.c_float
         L.ofo_kth_largest.argtypes = [f32p, C.c_int, C.c_int]
         L.ofo_log_sum_exp.restype = C.c_float
@@ -76,6 +78,12 @@ def default_opt(**kw):
 
 def crc32c(crc, bits, nbits):
     return int(lib().ofo_crc32c(crc & 0xFFFFFFFF, bits & 0xFFFFFFFF, nbits))
+
+
+def set_seed_state_mask(mask=0xFFFFFFFF):
+    """test knob: seed hashes from (state & mask); a narrow mask makes sequences share hashes.
+    Reset it (no argument) when done: the setting is process-wide."""
+    lib().ofo_set_seed_state_mask(mask & 0xFFFFFFFF)
 
 
 def kth_largest(values, k):

@@ -349,6 +349,73 @@ def test_five_column_input_equals_its_four_column_view(api, state_len, T, N):
     assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
 
 
+@pytest.mark.parametrize("state_len,T,N", [(4, 240, 6), (3, 300, 8), (5, 90, 2)])
+def test_duplicate_hashes_are_detected_and_merged_like_the_cpu_path(api, state_len, T, N):
+    """Beam elements whose sequences differ but whose hashes are equal (a CRC collision): forced
+    here by seeding the beam with hashes of (state & 15) on both sides.  A stay then finds several
+    equal hashes, and one step is claimed by two stays; the search has to notice that on its own
+    (no replay flag) and fall back to the CPU path's merge order."""
+    s16 = synth.crf_scores(T, N, state_len, seed={240: 2, 300: 4542, 90: 4332}[T])
+    kw = dict(q_scale=0.95, q_shift=-0.2)
+    plain = O.decode(s16.astype(np.float32), state_len, kw, nthreads=4)
+    O.set_seed_state_mask(15)
+    try:
+        ref = O.decode_from_tensors(s16.astype(np.float32), state_len, plain["bwd"], plain["post"], kw, nthreads=4)
+    finally:
+        O.set_seed_state_mask()
+    assert not np.array_equal(ref["moves"], plain["moves"]), "the shared hashes changed nothing: the case is too tame"
+    (mv, sq, qs), _ = gpu_from_tensors(api, s16, state_len, kw, plain["bwd"], plain["post"], debug_flags=2)
+    assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
+    (mv, sq, qs), _ = gpu_from_tensors(api, s16, state_len, kw, plain["bwd"], plain["post"], debug_flags=3)
+    assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]) and np.array_equal(qs, ref["qstring"])
+
+
+def test_two_threads_with_a_gpubuf_each_keep_their_own_settings(api):
+    """settings live in the gpubuf: a thread decoding with the hardware-exp scans and split kernels
+    does not change what a thread with the default settings gets, and the other way round"""
+    import threading
+    sl, T, N = 4, 500, 12
+    S = 4 ** sl
+    s16 = synth.crf_scores(T, N, sl, seed=314, chunk_scale=synth.stress_scale(N))
+    kw = dict(q_scale=0.95, q_shift=-0.2)
+    sc = api.upload_scores_to_hip(s16)
+    opt = api.DECODER_INIT(**kw)
+
+    def decode_with(mode, split, flags):
+        gb = api.GpuBuf(T, N, sl)
+        gb.set_scan_mode(mode)
+        gb.set_split_scans(split)
+        gb.set_debug_flags(flags)
+        out = api.openfish_decode_gpu(T, N, 4 * S, sc, sl, opt, gb)
+        return out, gb.tensor("bwd_NTC")
+
+    want = {"a": decode_with("two_tier", False, 0), "b": decode_with("fast", True, 1)}
+    assert not np.array_equal(want["a"][1], want["b"][1]), "the two settings should differ in the last bits of bwd"
+    got, errors = {"a": [], "b": []}, []
+
+    def worker(key, mode, split, flags):
+        try:
+            api.lib().set_device_hip(0)
+            for _ in range(6):
+                got[key].append(decode_with(mode, split, flags))
+        except Exception as e:  # surfaced below: an exception in a thread would otherwise pass silently
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=("a", "two_tier", False, 0)),
+               threading.Thread(target=worker, args=("b", "fast", True, 1))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+    for key in ("a", "b"):
+        assert len(got[key]) == 6
+        for (mv, sq, qs), bwd in got[key]:
+            assert np.array_equal(bwd, want[key][1])
+            assert np.array_equal(mv, want[key][0][0]) and np.array_equal(sq, want[key][0][1])
+            assert np.array_equal(qs, want[key][0][2])
+
+
 def test_constant_scores_closed_form(api):
     T, N, sl, c = 64, 3, 3, 0.75
     S = 4 ** sl
