@@ -167,8 +167,9 @@ __device__ __forceinline__ float log_sum_exp(float x, float y, const double *tab
 //   0.08  ln2f against ln 2, the rounding of the residual
 // together 3.64; the bound used is 4.0.  The result is settled when the distance from the
 // unrounded sum to the nearer rounding boundary of the result exceeds that bound (the residual of
-// the fused multiply-add, taken exactly with a second one); results that are zero, a power of two
-// or below 2^-102 in magnitude never count as settled.
+// the fused multiply-add, taken exactly with a second one).  Half an ulp is read from the exponent
+// of the next smaller float, which for a power of two is the binade below, where its nearer
+// boundary lies; results that are zero or below 2^-102 in magnitude never count as settled.
 __device__ __forceinline__ float log_sum_exp_estimate(float x, float y, bool &settled) {
     const float gap = fabsf(x - y);
     const float top = x > y ? x : y;
@@ -178,8 +179,8 @@ __device__ __forceinline__ float log_sum_exp_estimate(float x, float y, bool &se
     const float r = __builtin_fmaf(l2, kLn2, top);
     const float rho = __builtin_fmaf(l2, kLn2, -(r - top));
     const uint32_t rb = __float_as_uint(r);
-    const float half_ulp = __uint_as_float((rb & 0x7f800000u) - (24u << 23));
-    settled = (half_ulp - fabsf(rho) > 4.0f * 5.9604644775390625e-8f) && (rb & 0x007fffffu) != 0;
+    const float half_ulp = __uint_as_float(((rb & 0x7fffffffu) - ((24u << 23) + 1u)) & 0xff800000u);
+    settled = half_ulp - fabsf(rho) > 4.0f * 5.9604644775390625e-8f;
     return r;
 }
 

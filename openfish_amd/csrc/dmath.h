@@ -227,8 +227,10 @@ OFA_HD float lse5_cpu_rounding_tab(float v0, float v1, float v2, float v3, float
 // r~ is settled when no rounding boundary lies within eps of x~: with rho = x~ - r~ (exact up
 // to one rounding: r~ - m is exact by Sterbenz' lemma once |m| >= 3.3, and smaller |m| are
 // never settled because half an ulp of r~ is then below eps) and h = half an ulp of r~, the
-// distance from x~ to the nearer boundary is h - |rho|, unless r~ is a power of two, whose lower
-// boundary is only h/2 away: those (and zero) count as unsettled.
+// distance from x~ to the nearer boundary is at least h - |rho|.  A power of two has its lower
+// boundary only a quarter of its ulp away: h is read from the exponent of the next smaller
+// float, which is the binade below exactly for powers of two, so that one comparison serves
+// every case.  Values below 2^-102 (zero included) come out with h <= 0 and are never settled.
 // ---------------------------------------------------------------------------------------------
 OFA_HD float exp2_hw(float x) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -264,9 +266,10 @@ OFA_HD Lse5Estimate lse5_estimate(float v0, float v1, float v2, float v3, float 
     e.value = __builtin_fmaf(l2, kLn2, m);
     const float rho = __builtin_fmaf(l2, kLn2, -(e.value - m));
     const uint32_t rb = bits_of(e.value);
-    const float h = float_of((rb & 0x7f800000u) - (24u << 23));  // negative or huge-negative below 2^-102
+    // exponent field of the float below |r~|, lowered by 24; where that wraps, the sign bit survives the mask
+    const float h = float_of(((rb & 0x7fffffffu) - ((24u << 23) + 1u)) & 0xff800000u);
     const float eps = __builtin_fmaf(float_of(bits_of(s) & 0x7f800000u), kEps1, kEps0);
-    e.settled = (h - __builtin_fabsf(rho) > eps) && (rb & 0x007fffffu) != 0;
+    e.settled = h - __builtin_fabsf(rho) > eps;
     return e;
 }
 

@@ -207,13 +207,7 @@ __device__ __forceinline__ float lse5(float v0, float v1, float v2, float v3, fl
         return ofa::lse5_cpu_rounding_tab(v0, v1, v2, v3, v4, m, logtab.cells, logtab.series, logtab.expc);
     } else if constexpr (MODE == OFK_SCAN_TWO_TIER) {
         const ofa::Lse5Estimate e = ofa::lse5_estimate(v0, v1, v2, v3, v4, m);
-#if defined(OFK_EXPERIMENT_NO_RESOLVE)
-        return e.settled ? e.value : e.value + 0.0f * m;
-#elif defined(OFK_EXPERIMENT_BALLOT_ONLY)
-        return __builtin_amdgcn_ballot_w64(!e.settled) == 0x123456789ull ? m : e.value;
-#else
         return resolve_unsettled(e.value, e.sum, !e.settled, v0, v1, v2, v3, v4, m, logtab);
-#endif
     } else {
         float s = __builtin_amdgcn_exp2f((v0 - m) * kLog2e);
         s += __builtin_amdgcn_exp2f((v1 - m) * kLog2e);

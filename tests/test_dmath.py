@@ -103,11 +103,32 @@ def test_two_tier_estimate_is_never_wrongly_settled(lib, centre, spread, max_ope
 
 
 def test_two_tier_special_values_are_left_to_the_double_arithmetic(lib):
-    """results that are zero, a power of two or tiny never count as settled"""
+    """results that are zero or tiny never count as settled; a power of two may, and is then right"""
     cases = np.array([[0.0, -90.0, -90.0, -90.0, -90.0],      # exactly 0 + log(1 + tiny)
-                      [4096.0, 3000.0, 3000.0, 3000.0, 3000.0],  # a power of two
                       [1e-3, -1.0, -2.0, -3.0, -4.0],
-                      [-2.5, -2.5, -2.5, -2.5, -2.5]], np.float32)
+                      [-2.5, -2.5, -2.5, -2.5, -2.5],
+                      [4096.0, 3000.0, 3000.0, 3000.0, 3000.0]], np.float32)  # a power of two
     unsettled, mismatches = C.c_long(), C.c_long()
-    wrong = lib.two_tier_wrongly_settled(fptr(cases), cases.shape[0], C.byref(unsettled), C.byref(mismatches))
-    assert wrong == 0 and mismatches.value == 0 and unsettled.value == cases.shape[0]
+    wrong = lib.two_tier_wrongly_settled(fptr(cases[:3]), 3, C.byref(unsettled), C.byref(mismatches))
+    assert wrong == 0 and mismatches.value == 0 and unsettled.value == 3
+    wrong = lib.two_tier_wrongly_settled(fptr(cases), 4, C.byref(unsettled), C.byref(mismatches))
+    assert wrong == 0 and mismatches.value == 0
+
+
+@pytest.mark.parametrize("power", [4.0, 8.0, 64.0, 512.0, 4096.0, 32768.0, -8.0, -512.0])
+def test_two_tier_results_next_to_a_power_of_two(lib, power):
+    """the rounding boundary below a power of two is half as far away as the one above it: results
+    scattered closely around +-2^k (the sum is 1 + one more term, chosen so that max + log(sum)
+    lands within a few ulps of the power) must never be settled on the wrong side"""
+    rng = np.random.default_rng(int(abs(power)) + 5)
+    n = 300000
+    gap = rng.uniform(1e-3 + 4.0 * np.spacing(np.float32(abs(power))), np.log(2.0), n)  # power - max
+    big = power - gap
+    ulps = rng.uniform(-3.0, 3.0, n) * np.spacing(np.float32(abs(power)))
+    other = big + np.log(np.expm1(gap + ulps))          # exp(other - big) = exp(gap) - 1
+    v = np.stack([big, other, big - 200.0, big - 300.0, big - 400.0], axis=1).astype(np.float32)
+    unsettled, mismatches = C.c_long(), C.c_long()
+    wrong = lib.two_tier_wrongly_settled(fptr(v), n, C.byref(unsettled), C.byref(mismatches))
+    assert wrong == 0 and mismatches.value == 0
+    if abs(power) >= 64.0:  # below that, half an ulp is within the error bound and nothing is ever settled
+        assert unsettled.value < n  # some are settled: the case does exercise the settled branch
