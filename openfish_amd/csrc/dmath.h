@@ -210,19 +210,27 @@ OFA_HD float lse5_cpu_rounding_tab(float v0, float v1, float v2, float v3, float
 // s_cpu the fp32 running sum of the double exponentials.  The estimate forms
 //   t_i = RN32(d_i * c),  E_i = exp2(t_i),  s~ = fp32 running sum of E_i,  l2 = log2(s~),
 //   r~ = RN32(m + l2 * ln2f)          (one fused multiply-add)
-// and x~ = m + l2 * ln2f differs from x = m + ln s_cpu by at most eps, all terms in units of
-// 2^-24 = 5.96e-8:
-//   5.00  s_cpu against the exact sum S of the e^{d_i}: five roundings of at most half an ulp
-//         of a partial sum <= s
-//   4.00  s~ against the exact sum of the E_i: four fp32 additions
+// and x~ = m + l2 * ln2f differs from x = m + ln s_cpu by at most eps.  With s~ in
+// [2^k, 2^(k+1)) and all terms in units of 2^-24 = 5.96e-8:
+//   8.5 * 2^k / s   roundings of the two running sums.  s_cpu against the exact sum S of the
+//         e^{d_i}: the first term rounded to fp32 (half an ulp of a number <= 1: 0.5 absolute)
+//         and four additions, each off by at most half an ulp of a partial sum <= s, i.e. by 2^k
+//         absolute; s~ against the exact sum of the E_i: four fp32 additions, 2^k each.
+//         Relative to s that is (0.5 + 8 * 2^k) / s <= 8.5 * 2^k / s
 //   1.43 (S-1)/S   v_exp_f32: largest relative error found over every input in [-160, 0] is
-//         1.423 * 2^-24; the term with d = 0 is exactly 1
+//         1.423 * 2^-24; the term with d = 0 is exactly 1; (S-1)/S <= 0.5, 0.75, 0.8 for k = 0, 1, 2
 //   0.88  argument of exp2: t_i = d_i c (1 + p), |p| <= 2^-24 + 1.34e-8 (c rounded to fp32), a
 //         relative error |d_i| p of E_i; sum_i |d_i| e^{d_i} / S <= 0.718
 //   0.70 * 2^k  v_log_f32: largest absolute error found over every input in [1, 5.01] is
 //         1.0, 2.0, 4.0 * 2^-24 for s~ in [1,2), [2,4), [4,5.01]; times ln 2
 //   0.12  ln2f against ln 2 (1.9e-9 * l2), rounding of the residual below, second-order terms
-// i.e. 11.41, 12.46, 13.91 for the three binades of s~; eps below adds 3 %.
+// The last four add up to 2.415, 3.463, 4.914 for k = 0, 1, 2, all at most 1.38 + 1.045 * 2^k.
+// With mu = s~ / 2^(k+1) in [0.5, 1), 2^k / s = 1 / (2 mu) <= 1.5 - mu (the chord of a convex
+// function), so that
+//   eps = 14.13 - 8.5 mu + 1.045 * 2^k    (11.0 at s~ = 1, 6.7 just below 2, 12.0 at 2, ...)
+// is a bound, evaluated from the bits of s~ with two fused multiply-adds; the constants below
+// add 3 %.  The binade is read from s~ raised by 16 ulps: should s_cpu, within a dozen ulps
+// of s~, reach the next binade, where half an ulp is twice as large, s~ counts as being there too.
 //
 // r~ is settled when no rounding boundary lies within eps of x~: with rho = x~ - r~ (exact up
 // to one rounding: r~ - m is exact by Sterbenz' lemma once |m| >= 3.3, and smaller |m| are
@@ -259,7 +267,7 @@ OFA_HD Lse5Estimate lse5_estimate(float v0, float v1, float v2, float v3, float 
     s += exp2_hw((v2 - m) * kLog2e);
     s += exp2_hw((v3 - m) * kLog2e);
     s += exp2_hw((v4 - m) * kLog2e);
-    const float kEps0 = 6.35e-7f, kEps1 = 0.65e-7f;
+    const float kEps0 = 8.68e-7f, kEpsMu = 5.21e-7f, kEps1 = 6.42e-8f;
     const float l2 = log2_hw(s);
     Lse5Estimate e;
     e.sum = s;
@@ -268,7 +276,9 @@ OFA_HD Lse5Estimate lse5_estimate(float v0, float v1, float v2, float v3, float 
     const uint32_t rb = bits_of(e.value);
     // exponent field of the float below |r~|, lowered by 24; where that wraps, the sign bit survives the mask
     const float h = float_of(((rb & 0x7fffffffu) - ((24u << 23) + 1u)) & 0xff800000u);
-    const float eps = __builtin_fmaf(float_of(bits_of(s) & 0x7f800000u), kEps1, kEps0);
+    const uint32_t sb = bits_of(s) + 16u;
+    const float mu = float_of((sb & 0x007fffffu) | 0x3f000000u);
+    const float eps = __builtin_fmaf(mu, -kEpsMu, __builtin_fmaf(float_of(sb & 0x7f800000u), kEps1, kEps0));
     e.settled = h - __builtin_fabsf(rho) > eps;
     return e;
 }

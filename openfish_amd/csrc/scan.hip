@@ -139,10 +139,6 @@ struct LogArgs {
 // further trips (only the first few dozen time steps have that many: values are small there and
 // an ulp is tiny; the kernels run those steps with the double arithmetic throughout).
 #ifdef OFK_TIER_STATS
-__device__ unsigned long long g_tier_stats[4];  // wave-level calls, calls with unsettled lanes, trips, unsettled lanes
-#endif
-
-#ifdef OFK_TIER_STATS
 // build with -DOFK_TIER_STATS to count, per wave-level update of the two-tier scans: updates, updates
 // with unsettled lanes, second-tier trips, unsettled lanes (read with ofk_tier_stats)
 __device__ unsigned long long g_tier_stats[4];

@@ -132,3 +132,26 @@ def test_two_tier_results_next_to_a_power_of_two(lib, power):
     assert wrong == 0 and mismatches.value == 0
     if abs(power) >= 64.0:  # below that, half an ulp is within the error bound and nothing is ever settled
         assert unsettled.value < n  # some are settled: the case does exercise the settled branch
+
+
+@pytest.mark.parametrize("terms,centre", [(2, 300.0), (2, 3000.0), (4, 900.0), (4, 5000.0), (3, 2500.0)])
+def test_two_tier_sums_next_to_a_binade_of_the_sum(lib, terms, centre):
+    """sums of exponentials scattered closely around 2 and 4, where the ulp of the CPU path's
+    partial sums doubles: `terms` values within a few 1e-7 of the maximum (and, for three terms,
+    one a factor of two further down, which lands on 2 + 1/2 + ... as well as on sums just below
+    and above 2 and 4 through the scatter), the rest far below"""
+    rng = np.random.default_rng(terms * 1000 + int(centre))
+    n = 400000
+    top = (centre + rng.uniform(-40.0, 40.0, n)).astype(np.float32)
+    v = np.empty((n, 5), np.float64)
+    for k in range(5):
+        if k < terms:
+            v[:, k] = top.astype(np.float64) - np.abs(rng.normal(0.0, 3e-4 * (k > 0), n))
+        else:
+            v[:, k] = top.astype(np.float64) - rng.uniform(14.0, 40.0, n)
+    order = rng.permuted(np.tile(np.arange(5), (n, 1)), axis=1)   # the maximum in any position
+    v = np.take_along_axis(v, order, axis=1).astype(np.float32)
+    unsettled, mismatches = C.c_long(), C.c_long()
+    wrong = lib.two_tier_wrongly_settled(fptr(v), n, C.byref(unsettled), C.byref(mismatches))
+    assert wrong == 0 and mismatches.value == 0
+    assert unsettled.value < n
