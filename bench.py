@@ -302,7 +302,8 @@ def main():
         "vs_baseline": None, "dtype": "f32" if a.scan_mode == "fast" else "f32+f64", "data": "synthetic",
         "config": {"workload": "%s: state_len %d, S=%d, C=%d fp16 TNC (%d columns per state), T=%d, N=%d, beam 32, "
                                "beam_cut 100, blank 2.0" % (a.workload, state_len, S, C, a.columns, T, N),
-                   "scan_mode": a.scan_mode, "scans": "split" if a.split_scans else "one kernel", "seed": a.seed},
+                   "scan_mode": a.scan_mode, "scans": "one kernel" if mean["scan"] > 0 else "two kernels (backward, then forward + posterior beside the beam search)",
+                   "seed": a.seed},
         "roofline": roofline, "stages": stages, "other_scan_arrangement": other_split, "fast_scan_mode": fast_mode,
         "two_in_flight": overlap, "cpu_baseline": cpu,
     }))
