@@ -68,7 +68,8 @@ enum openfish_amd_scan_mode {
 
 /*
  * Backward scan (reference backward_scan src/decode_cpu.c:13-52, GPU twin
- * bwd_scan src/scan_hip.hip:9-58).  scores: device half [T][N][C], C = 4*S.
+ * bwd_scan src/scan_hip.hip:9-58).  scores: device half [T][N][C], C = 4*S, or 5*S with an
+ * unused blank value in front of the four of every state (all stages take both layouts).
  * bwd: device fp32 [N][T+1][S], row T is zero.
  */
 void openfish_amd_bwd_scan(int T, int N, int C, const void *scores, int state_len, float stay_score,

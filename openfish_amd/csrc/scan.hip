@@ -18,15 +18,22 @@
 //
 // Arithmetic follows the CPU path (reference src/decode_cpu.c:13-147): fp32
 // sums of state value and score, max, exp of the fp32 differences, running sum
-// in transition order, max + log(sum).  Two variants of that last step exist:
-//   precise: exp and log in double, the running sum rounded to fp32 after every
-//            term and one rounding of max + log(sum), i.e. the CPU path's own
-//            sequence of roundings (fp64 FMA issues at the fp32 rate on gfx950);
-//   fast   : v_exp_f32 / v_log_f32, within an ulp or two of the precise result.
+// in transition order, max + log(sum).  Three variants of that last step exist:
+//   precise : exp and log in double, the running sum rounded to fp32 after every
+//             term and one rounding of max + log(sum), i.e. the CPU path's own
+//             sequence of roundings (fp64 FMA issues at the fp32 rate on gfx950);
+//   fast    : v_exp_f32 / v_log_f32, within an ulp or two of the precise result;
+//   two-tier: the fast value wherever it provably rounds like the precise one (its
+//             distance to a rounding boundary exceeds a bound on its error), the
+//             precise arithmetic for the remaining lanes.  Same bits as precise.
 // State values reach several thousand, where one fp32 ulp is already 5e-4, and
 // the posterior is exp(fwd + bwd - const): a last-bit difference in a scan shows
-// up as a 5e-4 relative difference of a posterior.  The precise variant is the
-// default for that reason.
+// up as a 5e-4 relative difference of a posterior.  Two-tier is the default for
+// that reason; fast exists for measurements.
+//
+// Kernels: bwd_scan_kernel and fwd_post_kernel are the two sweeps one after the other;
+// scan_post_kernel runs both sweeps of a chunk in one workgroup, from both ends of the
+// chunk towards the middle and on to the other end, and is what a decode uses.
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -228,6 +235,19 @@ struct Shape {
     static constexpr int kQuarter = S / 4;
 };
 
+// The backward sweep keeps its state vector in LDS with the four quarters {c * S/4 ..} spaced
+// S/4 + kPad floats apart: a lane stores r + c * S/4, and with S/4 a multiple of the 64 banks
+// the lanes of a wave that differ only in c would all hit one bank.  16 floats of padding
+// spread them over all banks; reads of the contiguous quad {4r + b} stay 16-byte aligned.
+template <int S>
+struct BwdVec {
+    static constexpr int kQ = S / 4;
+    static constexpr int kPad = kQ % 64 == 0 ? 16 : 0;
+    static constexpr int kLen = S + 4 * kPad;
+    static __device__ __forceinline__ int at(int r, int c) { return r + c * (kQ + kPad); }  // state r + c * S/4, r < S/4
+    static __device__ __forceinline__ int of(int s) { return s + kPad * (s / kQ); }         // any state s
+};
+
 // x + (float)h for the fp16 value h in the low (HI = 0) or high half of a 32-bit register, in one
 // instruction: v_fma_mix_f32 converts the half operand on the fly, the product with 1.0 is
 // exact, so the result is the correctly rounded fp32 sum, bit for bit what v_cvt_f32_f16
@@ -383,7 +403,8 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
     constexpr int L = Sh::kLanes;
     constexpr int Q = Sh::kQuarter;
     constexpr int H = 4 / SPL;  // lanes sharing one quad
-    __shared__ __attribute__((aligned(16))) float vec[Sh::kChunks][2][S];
+    using Vec = BwdVec<S>;
+    __shared__ __attribute__((aligned(16))) float vec[Sh::kChunks][2][Vec::kLen];
     __shared__ __attribute__((aligned(16))) ofa::LogCell logcells[32];
     __shared__ __attribute__((aligned(16))) float tier_lanes[MODE == OFK_SCAN_TWO_TIER ? Sh::kThreads : 64];
     const int tid = threadIdx.x;
@@ -417,7 +438,7 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
 
     int buf = 0;
 #pragma unroll
-    for (int i = 0; i < SPL; ++i) vec[g][0][r + (c0 + i) * Q] = 0.f;
+    for (int i = 0; i < SPL; ++i) vec[g][0][Vec::at(r, c0 + i)] = 0.f;
     __syncthreads();  // the log table is shared by the whole group
 
     for (int done = 0; done < T; done += DEPTH) {
@@ -428,11 +449,11 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void bwd_scan_kernel(
                 const BwdRow<SPL> row = ring[k];
                 if (t - DEPTH >= 0) ring[k].load(sp + (size_t)(t - DEPTH) * row_stride);
                 chunk_sync<Sh::kMultiWave>();
-                const float4 nx = *reinterpret_cast<const float4 *>(&vec[g][buf][4 * r]);
+                const float4 nx = *reinterpret_cast<const float4 *>(&vec[g][buf][Vec::of(4 * r)]);
                 bwd_update<0, SPL, MODE>(a, nx, row, stay, logtab);
                 buf ^= 1;
 #pragma unroll
-                for (int i = 0; i < SPL; ++i) vec[g][buf][r + (c0 + i) * Q] = a[i];
+                for (int i = 0; i < SPL; ++i) vec[g][buf][Vec::at(r, c0 + i)] = a[i];
                 if (live) {
 #pragma unroll
                     for (int i = 0; i < SPL; ++i) out[(size_t)t * S + i * Q] = a[i];
@@ -624,7 +645,8 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
     constexpr int RW = Sh::kRoleWaves;
     constexpr int H4 = 4 / SPL;  // backward lanes sharing one quad
     constexpr int kWarmup = 32;  // time steps of either sweep evaluated in double before the two tiers take over
-    __shared__ __attribute__((aligned(16))) float vecB[Sh::kChunks][2][S];
+    using VecB = BwdVec<S>;
+    __shared__ __attribute__((aligned(16))) float vecB[Sh::kChunks][2][VecB::kLen];
     __shared__ __attribute__((aligned(16))) float vecF[Sh::kChunks][2][S];
     __shared__ float part[Sh::kChunks][2][2][RW];  // [chunk][direction][parity][wave]
     __shared__ float shift_of[Sh::kChunks];
@@ -662,7 +684,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
 #pragma unroll
         for (int i = 0; i < SPL; ++i) {
             a[i] = 0.f;
-            vecB[g][0][r + (c0 + i) * Q] = 0.f;
+            vecB[g][0][VecB::at(r, c0 + i)] = 0.f;
             if (live) bwd_blk[(size_t)T * S + st_lane + i * Q] = 0.f;
         }
         int buf = 0;
@@ -689,11 +711,11 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                     pre -= row_stride;
                 }
                 block_barrier_lds();
-                const float4 nx = *reinterpret_cast<const float4 *>(&vecB[g][buf][4 * r]);
+                const float4 nx = *reinterpret_cast<const float4 *>(&vecB[g][buf][VecB::of(4 * r)]);
                 bwd_update<0, SPL, M>(a, nx, row, stay, logtab);
                 buf ^= 1;
 #pragma unroll
-                for (int i = 0; i < SPL; ++i) vecB[g][buf][r + (c0 + i) * Q] = a[i];
+                for (int i = 0; i < SPL; ++i) vecB[g][buf][VecB::at(r, c0 + i)] = a[i];
                 if (live) {
 #pragma unroll
                     for (int i = 0; i < SPL; ++i) orow[st_lane + i * Q] = a[i];
@@ -754,13 +776,13 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                     }
                 }
                 prow -= S;
-                const float4 nx = *reinterpret_cast<const float4 *>(&vecB[g][buf][4 * r]);
+                const float4 nx = *reinterpret_cast<const float4 *>(&vecB[g][buf][VecB::of(4 * r)]);
                 bwd_update<0, SPL, MODE>(a, nx, row, stay, logtab);
                 buf ^= 1;
                 float total;
 #pragma unroll
                 for (int i = 0; i < SPL; ++i) {
-                    vecB[g][buf][r + (c0 + i) * Q] = a[i];
+                    vecB[g][buf][VecB::at(r, c0 + i)] = a[i];
                     e_prev[i] = __builtin_amdgcn_exp2f(((fv[i] + a[i]) - shift) * kLog2e);
                     total = i ? total + e_prev[i] : e_prev[i];
                 }
@@ -848,7 +870,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
         {
             const int bbuf = (T - H) & 1;  // where the backward lanes left bwd[H]
             FloatRun<SPL> bh;
-            bh.load(&vecB[g][bbuf][s0]);
+            bh.load(&vecB[g][bbuf][VecB::of(s0)]);
             float m = f[0] + bh.v[0];
 #pragma unroll
             for (int i = 1; i < SPL; ++i) m = fmaxf(m, f[i] + bh.v[i]);

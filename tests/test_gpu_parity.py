@@ -314,7 +314,8 @@ def test_enqueue_and_wait_with_two_batches_in_flight(api):
         del dev
 
 
-@pytest.mark.parametrize("state_len,T,N", [(3, 150, 5), (4, 90, 3), (5, 40, 2), (4, 333, 40), (3, 64, 9)])
+@pytest.mark.parametrize("state_len,T,N", [(3, 150, 5), (4, 90, 3), (5, 40, 2), (4, 333, 40), (3, 64, 9), (3, 1, 2), (4, 2, 1),
+                                           (5, 3, 1)])
 def test_five_column_input_equals_its_four_column_view(api, state_len, T, N):
     """C = 5*S: a blank column in front of the four step columns of every state, read where it
     lies by every kernel that takes scores; the blank values (poisoned here) are never looked at"""
