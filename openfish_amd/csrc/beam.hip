@@ -270,8 +270,6 @@ struct BeamRing {
 template <int S>
 struct BeamTrace {
     ofk_beam_slot_t slot[BeamCfg<S>::kTraceBlock][kW];
-    int32_t state[BeamCfg<S>::kTraceBlock];
-    uint8_t move[BeamCfg<S>::kTraceBlock];
 };
 template <int S, int COLS>
 struct __attribute__((aligned(16))) BeamLds {
@@ -317,8 +315,6 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     auto &row_b = lds[member].ring.row_b;
     BeamShared &sh = lds[member].sh;
     auto &trace = lds[member].trace.slot;
-    auto &trace_state = lds[member].trace.state;
-    auto &trace_move = lds[member].trace.move;
     const size_t row_stride = (size_t)N * COLS * S;
     const _Float16 *sc_n = scores + (size_t)n * COLS * S;
     const float *bw_n = bwd + (size_t)n * (size_t)(T + 1) * S;
@@ -711,11 +707,17 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     }
 
     // ---- traceback from slot 0 of the last block (src/beam_search.c:432-439) ----
+    // The chase itself is serial: one LDS read per time step, its address taken from the slot
+    // read before.  Everything else is kept off that chain: the slot of row k of a round of 64
+    // rows is parked in lane k (a compare and a select over the whole wave; instructions that
+    // run with one lane enabled were measured to take three to five times as long as with all
+    // 64), and after the round every lane unpacks its own row and the wave stores 64 states and
+    // moves side by side.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     int32_t *st_out = states + (size_t)n * T;
     uint8_t *mv_out = moves + (size_t)n * T;
-    int cursor = 0;
+    uint32_t cursor = 0;  // the same in every lane
     for (int hi_t = T; hi_t > 0; hi_t -= TB) {
         const int lo_t = hi_t > TB ? hi_t - TB : 0;  // rows lo_t+1 .. hi_t
         const int rows = hi_t - lo_t;
@@ -723,18 +725,19 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         uint4 *dst = reinterpret_cast<uint4 *>(&trace[0][0]);
         for (int x = lane; x < rows * 4; x += 64) dst[x] = src[x];  // 64 bytes per row
         wave_fence();
-        for (int r = rows - 1; r >= 0; --r) {
-            const uint32_t e = trace[r][cursor];
-            if (lane == 0) {
-                trace_state[r] = (int32_t)(e & 1023u);
-                trace_move[r] = (e >> 15) ? 0 : 1;
+        for (int top = rows; top > 0; top -= 64) {
+            const int first = __builtin_amdgcn_readfirstlane(top > 64 ? top - 64 : 0);  // this round: rows first .. top-1, newest first
+            uint32_t mine = 0;
+            for (int r = top - 1; r >= first; --r) {
+                const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)trace[r][cursor]);
+                mine = lane == r - first ? e : mine;
+                cursor = (e >> 10) & 31u;
             }
-            cursor = (int)((e >> 10) & 31u);
-        }
-        wave_fence();
-        for (int x = lane; x < rows; x += 64) {
-            st_out[lo_t + x] = trace_state[x];
-            mv_out[lo_t + x] = (lo_t + x == 0) ? (uint8_t)1 : trace_move[x];
+            const int t = lo_t + first + lane;
+            if (first + lane < top) {
+                st_out[t] = (int32_t)(mine & 1023u);
+                mv_out[t] = (t == 0 || !(mine >> 15)) ? (uint8_t)1 : (uint8_t)0;
+            }
         }
         wave_fence();
     }
