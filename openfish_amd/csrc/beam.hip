@@ -111,6 +111,20 @@ __device__ __forceinline__ int wave_sum_i(int x) {
            __builtin_amdgcn_readlane(x, 32) + __builtin_amdgcn_readlane(x, 48);
 }
 __device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
+// per lane: yes where the lane's bit of a wave-wide mask is set, no elsewhere; the mask goes into
+// the select as it is (a comparison result the wave already holds in scalar registers)
+__device__ __forceinline__ int pick_by_bit(uint64_t mask, int yes, int no) {
+    int r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(mask));
+    return r;
+}
+// x + (the lane's bit of mask), one add-with-carry
+__device__ __forceinline__ int add_bit_of(int x, uint64_t mask) {
+    int r;
+    uint64_t carry;
+    asm("v_addc_co_u32_e64 %0, %1, %2, 0, %3" : "=v"(r), "=&s"(carry) : "v"(x), "s"(mask));
+    return r;
+}
 __device__ __forceinline__ int popc64(uint64_t x) { return __builtin_popcountll(x); }
 // Any lane with a non-zero word.  The ballot of a plain comparison is the comparison's own lane
 // mask; the ballot of a combined condition would take a detour through two more vector
@@ -240,7 +254,7 @@ struct BeamCfg {
 struct __attribute__((aligned(16))) Elem {
     uint32_t hash;
     float score;    // candidate score, guide term of its state included
-    uint32_t info;  // state | prev << 16 | stay << 21
+    uint32_t info;  // state | prev << 10 | stay << 15: the 16-bit slot the traceback reads
     float rest;     // score minus that guide term: what the next time step starts from
 };
 // mailbox of one step candidate (index 4i+b): what a stay that merged with it leaves behind
@@ -427,7 +441,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         score = e.score;
         info = e.info;
     }
-    int state = (int)(info & 0xFFFFu);
+    int state = (int)(info & 1023u);
     int w = kW;
     ofk_beam_slot_t *bv = beam + (size_t)n * (size_t)(T + 1) * kW;
     bv[i] = (ofk_beam_slot_t)state;
@@ -436,6 +450,10 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     // throughput-bound waves (the forward scan runs at the same time) it should win the
     // issue arbitration.
     __builtin_amdgcn_s_setprio(3);
+    // Only the even lane of a pair carries the element's stay.  The odd lane adds -FLT_MAX instead of
+    // the stay score, so that its stay candidate is -FLT_MAX (or -inf once the element is dead):
+    // it never passes a cut and never wins a maximum, without a select in every time step.
+    const float stay_h = h == 0 ? stay : -FLT_MAX;
     int rows_ready = 0;  // last value seen of the loader's counter; it is usually several rows ahead
     const int b0 = 2 * h;
     // What a time step reads from LDS depends only on the beam it starts from, so it is
@@ -475,7 +493,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         const float r1 = (float)r1h;
         float c0 = (score + r0) + g01.x;
         float c1 = (score + r1) + g01.y;
-        float cs = (score + stay) + gst;
+        float cs = (score + stay_h) + gst;
         publish(&sh.consumed, t + 1);  // everything this step needs of row t is in registers
         const uint32_t h0 = crc2(hash, (uint32_t)b0);
         const uint32_t h1 = h0 ^ kTab1;  // crc2(hash, b0 + 1): b0 is even, so only bit 0 of the table index flips
@@ -600,8 +618,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
 
         // cut-off (src/beam_search.c:320-381)
         // Dead lanes carry -FLT_MAX as their score, which absorbs whatever is added: their candidates
-        // are -FLT_MAX exactly, and so is the stay of the upper half from here on.
-        cs = h == 0 ? cs : -FLT_MAX;
+        // are -FLT_MAX exactly (the stay of an odd lane: -FLT_MAX or -inf, see stay_h).
         float best;
         asm("v_max3_f32 %0, %1, %2, %3" : "=v"(best) : "v"(c0), "v"(c1), "v"(cs));
         best = wave_max(best);
@@ -609,6 +626,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         float cut = best - log_cut;  // may be -FLT_MAX (no cut at all): mask the dead lanes
         uint64_t k0 = ballot(c0 >= cut) & vm, k1 = ballot(c1 >= cut) & vm, ks = ballot(cs >= cut) & vs;
         int kept = popc64(k0) + popc64(k1) + popc64(ks);
+        bool overfull = false;  // more candidates than the width pass the final cut (the same in every lane)
         if (kept > kW) {
             // Bisection between the cut and the best score.  Every cut tried in here lies above
             // (-FLT_MAX + best) / 2, so dead lanes and dropped candidates never pass and the
@@ -637,7 +655,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 ks = ballot(cs >= cut);
                 kept = popc64(k0) + popc64(k1) + popc64(ks);
             }
-            if (kept > kW) kept = kW;
+            overfull = kept > kW;
+            if (overfull) kept = kW;
         }
 
         // survivors in candidate order: steps (i, b) by i then b, then stays by i
@@ -647,23 +666,31 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 return (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
                                                       __builtin_amdgcn_mbcnt_lo((uint32_t)mask, (uint32_t)start));
             };
-            const bool keep0 = valid && c0 >= cut, keep1 = valid && c1 >= cut;  // this lane's bits of k0, k1
-            const bool keeps = valid && h == 0 && cs >= cut;                      // and of ks
+            // k0, k1 and ks hold this lane's own verdicts at its bit (dead lanes and the stays of the odd
+            // lanes never pass): the masks select directly, nothing is compared again
             const int rank0 = lower(k1, lower(k0, 0));
-            const int rank1 = rank0 + (keep0 ? 1 : 0);
+            const int rank1 = add_bit_of(rank0, k0);
             const int ranks = lower(ks, popc64(k0) + popc64(k1));
-            const uint32_t from = (uint32_t)i << 16;
-            // every lane stores all three of its candidates, the ones that are dropped into the
-            // dump slot: no branches and no exec masking on the path from the cut-off to the next beam
-            const int slot0 = min(keep0 ? rank0 : kW, kW);
-            const int slot1 = min(keep1 ? rank1 : kW, kW);
-            const int slots = min(keeps ? ranks : kW, kW);
+            const uint32_t from = (uint32_t)i << 10;
+            // every lane stores all three of its candidates, the ones that are dropped into the dump
+            // slot: no exec masking on the path from the cut-off to the next beam.  Kept candidates
+            // beyond the width exist only after the ten-guess exit of the bisection; a branch that is
+            // almost never taken sends them to the dump slot as well.
+            int slot0 = pick_by_bit(k0, rank0, kW);
+            int slot1 = pick_by_bit(k1, rank1, kW);
+            int slots = pick_by_bit(ks, ranks, kW);
+            if (overfull) {
+                asm volatile("");  // keeps this a branch instead of three selects on every step
+                slot0 = min(slot0, kW);
+                slot1 = min(slot1, kW);
+                slots = min(slots, kW);
+            }
             sh.hash[slot0] = h0;
             sh.elem[slot0] = Elem{h0, c0, (uint32_t)(lo4 + b0) | from, c0 - g01.x};
             sh.hash[slot1] = h1;
             sh.elem[slot1] = Elem{h1, c1, (uint32_t)(lo4 + b0 + 1) | from, c1 - g01.y};
             sh.hash[slots] = hash;
-            sh.elem[slots] = Elem{hash, cs, (uint32_t)state | from | (1u << 21), cs - gst};
+            sh.elem[slots] = Elem{hash, cs, (uint32_t)state | from | (1u << 15), cs - gst};
             wave_fence();
         }
         w = kept;
@@ -677,7 +704,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             info = in ? e.info : 0u;
             rest = in ? e.rest : -FLT_MAX;
         }
-        state = (int)(info & 0xFFFFu);
+        state = (int)(info & 1023u);
         if (t + 1 < T) fetch_row(t + 1);
 
         // last block: the best survivor goes to slot 0 (src/beam_search.c:398-414)
@@ -693,7 +720,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 const float re0 = lane_f(rest, 0), rea = lane_f(rest, arg_lane);
                 if (i == 0) { hash = hasha; info = ina; rest = rea; }
                 if (i == arg) { hash = hash0; info = in0; rest = re0; }
-                state = (int)(info & 0xFFFFu);
+                state = (int)(info & 1023u);
             }
         }
 
@@ -703,7 +730,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // both halves hold the same element and store the same slot; slots past the width are never
         // followed by the traceback
         bv[(size_t)(t + 1) * kW + i] =
-            (ofk_beam_slot_t)((uint32_t)state | (((info >> 16) & 31u) << 10) | (((info >> 21) & 1u) << 15));
+            (ofk_beam_slot_t)info;
     }
 
     // ---- traceback from slot 0 of the last block (src/beam_search.c:432-439) ----
