@@ -102,6 +102,50 @@ __device__ __forceinline__ float wave_max(float x) {
         : "+v"(x));
     return lane_f(x, 63);
 }
+// What a lane will store for its three candidates once their ranks are known, worked out in the
+// wait states of the wave maximum: a wave that is alone on its SIMD pays a full issue slot (about
+// eight cycles) for every s_nop, so the two idle cycles each rotate-and-max step needs after its
+// source was written are filled with instructions that had to be issued anyway.
+//   h0 = crc2(hash, b0), h1 = crc2(hash, b0 + 1) = h0 ^ kTab1   (b0 is even)
+//   info0 = (lo4 + b0) | from, info1 = info0 | 1, infos = state | from | stay bit
+//   rest = candidate score minus its guide term
+struct NextRecords {
+    uint32_t h0, h1, info0, info1, infos;
+    float rest0, rest1, rests;
+};
+__device__ __forceinline__ float wave_max_beside_records(float x, NextRecords &n, uint32_t hash, uint32_t b0,
+                                                         uint32_t state_from_stay, uint32_t lo4b0_from, float c0,
+                                                         float c1, float cs, float g0, float g1, float gs) {
+    uint32_t t0, t1;
+    asm volatile(
+        "v_xor_b32 %[t0], %[hash], %[b0]\n\t"
+        "v_sub_f32 %[r0], %[c0], %[g0]\n\t"
+        "v_max_f32_dpp %[x], %[x], %[x] row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
+        "v_bfe_i32 %[t1], %[t0], 1, 1\n\t"
+        "v_bfe_i32 %[t0], %[t0], 0, 1\n\t"
+        "v_max_f32_dpp %[x], %[x], %[x] row_ror:4 row_mask:0xf bank_mask:0xf\n\t"
+        "v_and_b32 %[t1], %[tab2], %[t1]\n\t"
+        "v_and_b32 %[t0], %[tab1], %[t0]\n\t"
+        "v_max_f32_dpp %[x], %[x], %[x] row_ror:2 row_mask:0xf bank_mask:0xf\n\t"
+        "v_xor_b32 %[t0], %[t0], %[t1]\n\t"
+        "v_lshrrev_b32 %[t1], 2, %[hash]\n\t"
+        "v_max_f32_dpp %[x], %[x], %[x] row_ror:1 row_mask:0xf bank_mask:0xf\n\t"
+        "v_xor_b32 %[h0], %[t0], %[t1]\n\t"
+        "v_sub_f32 %[r1], %[c1], %[g1]\n\t"
+        "v_max_f32_dpp %[x], %[x], %[x] row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "v_xor_b32 %[h1], %[tab1], %[h0]\n\t"
+        "v_sub_f32 %[rs], %[cs], %[gs]\n\t"
+        "v_max_f32_dpp %[x], %[x], %[x] row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "v_or_b32 %[i1], 1, %[i0]\n\t"
+        "s_nop 0"
+        : [x] "+v"(x), [t0] "=&v"(t0), [t1] "=&v"(t1), [h0] "=&v"(n.h0), [h1] "=&v"(n.h1), [i1] "=&v"(n.info1),
+          [r0] "=&v"(n.rest0), [r1] "=&v"(n.rest1), [rs] "=&v"(n.rests)
+        : [hash] "v"(hash), [b0] "v"(b0), [tab1] "s"(kTab1), [tab2] "s"(kTab2), [i0] "v"(lo4b0_from), [c0] "v"(c0),
+          [c1] "v"(c1), [cs] "v"(cs), [g0] "v"(g0), [g1] "v"(g1), [gs] "v"(gs));
+    n.info0 = lo4b0_from;
+    n.infos = state_from_stay;
+    return lane_f(x, 63);
+}
 __device__ __forceinline__ int wave_sum_i(int x) {
     x += __builtin_amdgcn_update_dpp(0, x, 0x128, 0xF, 0xF, true);
     x += __builtin_amdgcn_update_dpp(0, x, 0x124, 0xF, 0xF, true);
@@ -454,6 +498,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     // the stay score, so that its stay candidate is -FLT_MAX (or -inf once the element is dead):
     // it never passes a cut and never wins a maximum, without a select in every time step.
     const float stay_h = h == 0 ? stay : -FLT_MAX;
+    const uint32_t from = (uint32_t)i << 10, from_stay = from | (1u << 15);  // the element's index as "prev" of its candidates
     int rows_ready = 0;  // last value seen of the loader's counter; it is usually several rows ahead
     const int b0 = 2 * h;
     // What a time step reads from LDS depends only on the beam it starts from, so it is
@@ -495,8 +540,6 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         float c1 = (score + r1) + g01.y;
         float cs = (score + stay_h) + gst;
         publish(&sh.consumed, t + 1);  // everything this step needs of row t is in registers
-        const uint32_t h0 = crc2(hash, (uint32_t)b0);
-        const uint32_t h1 = h0 ^ kTab1;  // crc2(hash, b0 + 1): b0 is even, so only bit 0 of the table index flips
         SlotRec *my_rec = &sh.rec[4 * i + b0];
 
         // which previous element j has hash_j == crc^-1(hash_i, last base of i)
@@ -621,7 +664,9 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // are -FLT_MAX exactly (the stay of an odd lane: -FLT_MAX or -inf, see stay_h).
         float best;
         asm("v_max3_f32 %0, %1, %2, %3" : "=v"(best) : "v"(c0), "v"(c1), "v"(cs));
-        best = wave_max(best);
+        NextRecords next;
+        best = wave_max_beside_records(best, next, hash, (uint32_t)b0, (uint32_t)state | from_stay,
+                                       (uint32_t)(lo4 + b0) | from, c0, c1, cs, g01.x, g01.y, gst);
 
         float cut = best - log_cut;  // may be -FLT_MAX (no cut at all): mask the dead lanes
         uint64_t k0 = ballot(c0 >= cut) & vm, k1 = ballot(c1 >= cut) & vm, ks = ballot(cs >= cut) & vs;
@@ -671,7 +716,6 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const int rank0 = lower(k1, lower(k0, 0));
             const int rank1 = add_bit_of(rank0, k0);
             const int ranks = lower(ks, popc64(k0) + popc64(k1));
-            const uint32_t from = (uint32_t)i << 10;
             // every lane stores all three of its candidates, the ones that are dropped into the dump
             // slot: no exec masking on the path from the cut-off to the next beam.  Kept candidates
             // beyond the width exist only after the ten-guess exit of the bisection; a branch that is
@@ -685,12 +729,12 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 slot1 = min(slot1, kW);
                 slots = min(slots, kW);
             }
-            sh.hash[slot0] = h0;
-            sh.elem[slot0] = Elem{h0, c0, (uint32_t)(lo4 + b0) | from, c0 - g01.x};
-            sh.hash[slot1] = h1;
-            sh.elem[slot1] = Elem{h1, c1, (uint32_t)(lo4 + b0 + 1) | from, c1 - g01.y};
+            sh.hash[slot0] = next.h0;
+            sh.elem[slot0] = Elem{next.h0, c0, next.info0, next.rest0};
+            sh.hash[slot1] = next.h1;
+            sh.elem[slot1] = Elem{next.h1, c1, next.info1, next.rest1};
             sh.hash[slots] = hash;
-            sh.elem[slots] = Elem{hash, cs, (uint32_t)state | from | (1u << 15), cs - gst};
+            sh.elem[slots] = Elem{hash, cs, next.infos, next.rests};
             wave_fence();
         }
         w = kept;
