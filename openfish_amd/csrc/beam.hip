@@ -109,15 +109,20 @@ __device__ __forceinline__ float wave_max(float x) {
 //   h0 = crc2(hash, b0), h1 = crc2(hash, b0 + 1) = h0 ^ kTab1   (b0 is even)
 //   info0 = (lo4 + b0) | from, info1 = info0 | 1, infos = state | from | stay bit
 //   rest = candidate score minus its guide term
+// The lane maximum (one v_max3) opens the block and the read of lane 63, where the six steps leave
+// the wave's maximum, closes it, each with its own wait states filled the same way.
 struct NextRecords {
     uint32_t h0, h1, info0, info1, infos;
     float rest0, rest1, rests;
 };
-__device__ __forceinline__ float wave_max_beside_records(float x, NextRecords &n, uint32_t hash, uint32_t b0,
-                                                         uint32_t state_from_stay, uint32_t lo4b0_from, float c0,
-                                                         float c1, float cs, float g0, float g1, float gs) {
-    uint32_t t0, t1;
+__device__ __forceinline__ float wave_max_beside_records(float c0, float c1, float cs, NextRecords &n, uint32_t hash,
+                                                         uint32_t b0, uint32_t state, uint32_t from_stay,
+                                                         uint32_t lo4b0, uint32_t from, float g0, float g1,
+                                                         float gs) {
+    uint32_t t0, t1, best;
+    float x;
     asm volatile(
+        "v_max3_f32 %[x], %[c0], %[c1], %[cs]\n\t"
         "v_xor_b32 %[t0], %[hash], %[b0]\n\t"
         "v_sub_f32 %[r0], %[c0], %[g0]\n\t"
         "v_max_f32_dpp %[x], %[x], %[x] row_ror:8 row_mask:0xf bank_mask:0xf\n\t"
@@ -136,15 +141,18 @@ __device__ __forceinline__ float wave_max_beside_records(float x, NextRecords &n
         "v_xor_b32 %[h1], %[tab1], %[h0]\n\t"
         "v_sub_f32 %[rs], %[cs], %[gs]\n\t"
         "v_max_f32_dpp %[x], %[x], %[x] row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "v_or_b32 %[i0], %[lo4b0], %[from]\n\t"
+        "v_or_b32 %[is], %[state], %[fromstay]\n\t"
+        "v_readlane_b32 %[best], %[x], 63\n\t"
         "v_or_b32 %[i1], 1, %[i0]\n\t"
         "s_nop 0"
-        : [x] "+v"(x), [t0] "=&v"(t0), [t1] "=&v"(t1), [h0] "=&v"(n.h0), [h1] "=&v"(n.h1), [i1] "=&v"(n.info1),
-          [r0] "=&v"(n.rest0), [r1] "=&v"(n.rest1), [rs] "=&v"(n.rests)
-        : [hash] "v"(hash), [b0] "v"(b0), [tab1] "s"(kTab1), [tab2] "s"(kTab2), [i0] "v"(lo4b0_from), [c0] "v"(c0),
-          [c1] "v"(c1), [cs] "v"(cs), [g0] "v"(g0), [g1] "v"(g1), [gs] "v"(gs));
-    n.info0 = lo4b0_from;
-    n.infos = state_from_stay;
-    return lane_f(x, 63);
+        : [x] "=&v"(x), [best] "=&s"(best), [t0] "=&v"(t0), [t1] "=&v"(t1), [h0] "=&v"(n.h0), [h1] "=&v"(n.h1),
+          [i0] "=&v"(n.info0), [i1] "=&v"(n.info1), [is] "=&v"(n.infos), [r0] "=&v"(n.rest0), [r1] "=&v"(n.rest1),
+          [rs] "=&v"(n.rests)
+        : [hash] "v"(hash), [b0] "v"(b0), [tab1] "s"(kTab1), [tab2] "s"(kTab2), [lo4b0] "v"(lo4b0), [from] "v"(from),
+          [state] "v"(state), [fromstay] "v"(from_stay), [c0] "v"(c0), [c1] "v"(c1), [cs] "v"(cs), [g0] "v"(g0),
+          [g1] "v"(g1), [gs] "v"(gs));
+    return __uint_as_float(best);
 }
 __device__ __forceinline__ int wave_sum_i(int x) {
     x += __builtin_amdgcn_update_dpp(0, x, 0x128, 0xF, 0xF, true);
@@ -170,13 +178,6 @@ __device__ __forceinline__ int add_bit_of(int x, uint64_t mask) {
     return r;
 }
 __device__ __forceinline__ int popc64(uint64_t x) { return __builtin_popcountll(x); }
-// Any lane with a non-zero word.  The ballot of a plain comparison is the comparison's own lane
-// mask; the ballot of a combined condition would take a detour through two more vector
-// instructions, so callers fold their condition into one integer first.
-__device__ __forceinline__ bool any_nonzero(uint32_t word) {
-    asm("" : "+v"(word));  // keeps the compiler from taking the word apart into its conditions again
-    return ballot(word != 0u) != 0;
-}
 
 __device__ __forceinline__ void wave_fence() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -533,6 +534,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         const bool valid = i < w;
         const uint64_t vm = ballot(valid);          // live elements, both halves
         const uint64_t vs = vm & 0x5555555555555555ull;  // their stay candidates sit on the even lanes
+        const uint64_t odd_base = ballot((state & 1) != 0);  // lanes whose element ends in base 1 or 3
         const int lo4 = (state << 2) & (S - 1);
         const float r0 = (float)r0h;
         const float r1 = (float)r1h;
@@ -585,14 +587,18 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 m |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1 /* quad_perm:[1,0,3,2] */, 0xF, 0xF, true);
             }
             const uint32_t live = w >= 32 ? 0xFFFFFFFFu : ((1u << w) - 1u);
-            match = valid ? (m & live) : 0u;
+            match = m & live;  // of a dead lane: leftovers, masked out below
         }
 
         // merge stays with the step spelling the same sequence (src/beam_search.c:281-316).
         // The stay's lane fetches the step's score from the lane that holds it, folds the two,
         // keeps its half of the outcome and leaves the step's half in the step's mailbox.
-        const bool mine = h == 0 && match != 0;
-        if (any_nonzero(h == 0 ? match : 0u)) {
+        // Conditions that hold per lane are kept as wave-wide masks in scalar registers and combined
+        // there; a select then takes its mask as it is.  (A condition put together from vector
+        // instructions right before its use costs the wait states between a compare and its reader,
+        // and a wave that is alone on its SIMD pays a whole issue slot for each.)
+        const uint64_t mine_mask = ballot(match != 0u) & vs;  // live even lanes whose stay has a partner
+        if (mine_mask != 0) {
             const uint32_t now = (uint32_t)(t + 1);
             const uint32_t mytag = (now << 5) | (uint32_t)i;
             const int j = __builtin_ctz(match | 0x80000000u) & 31;
@@ -600,18 +606,19 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const int holder = (2 * j + (bi >> 1)) << 2;  // the lane with element j and base bi, as a byte index
             const float o0 = __int_as_float(__builtin_amdgcn_ds_bpermute(holder, __float_as_int(c0)));
             const float o1 = __int_as_float(__builtin_amdgcn_ds_bpermute(holder, __float_as_int(c1)));
-            const float other = (bi & 1) ? o1 : o0;
-            const bool stay_wins = cs > other;
+            const float other = __int_as_float(pick_by_bit(odd_base, __float_as_int(o1), __float_as_int(o0)));
+            const uint64_t stay_wins = ballot(cs > other);
             // every lane goes through the fold and the mailbox, lanes without a merge with whatever
             // their registers hold and the dump slot as target: no exec masking on the way
             // the fold from hardware exp/log where that provably rounds like the CPU path's double
             // arithmetic (all but a few merges in a thousand at usual score magnitudes)
             bool settled;
             float folded = log_sum_exp_estimate(cs, other, settled);
-            if (any_nonzero(mine && !settled ? 1u : 0u)) folded = log_sum_exp(cs, other, lse);
-            const int target = mine ? 4 * j + bi : 4 * kW;
-            *reinterpret_cast<uint2 *>(&sh.rec[target]) =
-                make_uint2(mytag, __float_as_uint(stay_wins ? -FLT_MAX : folded));
+            if ((ballot(!settled) & mine_mask) != 0) folded = log_sum_exp(cs, other, lse);
+            const int target = pick_by_bit(mine_mask, 4 * j + bi, 4 * kW);
+            const float cs_merged = __int_as_float(pick_by_bit(stay_wins, __float_as_int(folded), __float_as_int(-FLT_MAX)));
+            *reinterpret_cast<uint2 *>(&sh.rec[target]) = make_uint2(
+                mytag, (uint32_t)pick_by_bit(stay_wins, __float_as_int(-FLT_MAX), __float_as_int(folded)));
             wave_fence();
             uint32_t claimed = sh.rec[target].tag;
             uint2 box0 = *reinterpret_cast<const uint2 *>(&my_rec[0]);
@@ -620,8 +627,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             // sink the mailbox reads below the branch that follows)
             asm volatile("" : "+v"(claimed), "+v"(box0.x), "+v"(box0.y), "+v"(box1.x), "+v"(box1.y));
             // odd: a stay with several equal hashes, or a step claimed by two stays
-            const uint32_t odd = mine ? ((match & (match - 1)) | (claimed ^ mytag)) : 0u;
-            if (any_nonzero(odd) || (flags & 1)) {
+            const uint32_t odd = (match & (match - 1)) | (claimed ^ mytag);
+            if ((ballot(odd != 0u) & mine_mask) != 0 || (flags & 1)) {
                 // A stay with several equal hashes, or a step claimed by two stays (only
                 // possible after a CRC collision): replay the merges one by one in the
                 // CPU path's order, from the scores as they were before any merge.
@@ -653,20 +660,30 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 c1 = my_rec[1].step;
             } else {
                 // of every matched pair one side carries the folded score on, the other is dropped
-                if (mine) cs = stay_wins ? folded : -FLT_MAX;
-                if ((box0.x >> 5) == now) c0 = __uint_as_float(box0.y);
-                if ((box1.x >> 5) == now) c1 = __uint_as_float(box1.y);
+                // (the two compares first, the stay's own select between them and the selects that read
+                // their masks: two instructions lie between every compare and its reader)
+                uint32_t tag0, tag1;
+                uint64_t hit0, hit1;
+                asm("v_lshrrev_b32 %[t0], 5, %[b0x]\n\t"
+                    "v_lshrrev_b32 %[t1], 5, %[b1x]\n\t"
+                    "v_cmp_eq_u32_e64 %[m0], %[now], %[t0]\n\t"
+                    "v_cmp_eq_u32_e64 %[m1], %[now], %[t1]\n\t"
+                    "v_cndmask_b32_e64 %[cs], %[cs], %[csm], %[mine]\n\t"
+                    "v_cndmask_b32_e64 %[c0], %[c0], %[b0y], %[m0]\n\t"
+                    "v_cndmask_b32_e64 %[c1], %[c1], %[b1y], %[m1]"
+                    : [c0] "+v"(c0), [c1] "+v"(c1), [cs] "+v"(cs), [t0] "=&v"(tag0), [t1] "=&v"(tag1),
+                      [m0] "=&s"(hit0), [m1] "=&s"(hit1)
+                    : [b0x] "v"(box0.x), [b1x] "v"(box1.x), [b0y] "v"(box0.y), [b1y] "v"(box1.y), [now] "s"(now),
+                      [csm] "v"(cs_merged), [mine] "s"(mine_mask));
             }
         }
 
         // cut-off (src/beam_search.c:320-381)
         // Dead lanes carry -FLT_MAX as their score, which absorbs whatever is added: their candidates
         // are -FLT_MAX exactly (the stay of an odd lane: -FLT_MAX or -inf, see stay_h).
-        float best;
-        asm("v_max3_f32 %0, %1, %2, %3" : "=v"(best) : "v"(c0), "v"(c1), "v"(cs));
         NextRecords next;
-        best = wave_max_beside_records(best, next, hash, (uint32_t)b0, (uint32_t)state | from_stay,
-                                       (uint32_t)(lo4 + b0) | from, c0, c1, cs, g01.x, g01.y, gst);
+        const float best = wave_max_beside_records(c0, c1, cs, next, hash, (uint32_t)b0, (uint32_t)state, from_stay,
+                                                   (uint32_t)(lo4 + b0), from, g01.x, g01.y, gst);
 
         float cut = best - log_cut;  // may be -FLT_MAX (no cut at all): mask the dead lanes
         uint64_t k0 = ballot(c0 >= cut) & vm, k1 = ballot(c1 >= cut) & vm, ks = ballot(cs >= cut) & vs;
