@@ -550,11 +550,34 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const uint32_t want = crc2_inverse(hash, (uint32_t)state & 3u);
             // Bit k of m says whether hash k of this half equals `want`.  Each comparison is
             // shifted into an accumulator with an add-with-carry (a = 2a + equal), two
-            // instructions per hash.  Two vectors of four hashes go through one block: the eight
-            // comparisons first, then the adds alternating between the vectors' accumulators, so
-            // that no instruction waits for the one before it.
-            auto eight = [&](const uint4 &x, const uint4 &y, uint32_t &ax, uint32_t &ay) {
+            // instructions per hash.  The low accumulator takes hashes 7..0, the high one hashes
+            // 15..8, eight comparisons at a time and the adds alternating between the two, so
+            // that no instruction waits for the one before it; each accumulator starts from the
+            // constant zero in its first add.
+            uint32_t lo8, hi8;
+            {
                 uint64_t e0, e1, e2, e3, f0, f1, f2, f3, carry;
+                asm("v_cmp_eq_u32_e64 %[e3], %[w], %[x3]\n\t"
+                    "v_cmp_eq_u32_e64 %[f3], %[w], %[y3]\n\t"
+                    "v_cmp_eq_u32_e64 %[e2], %[w], %[x2]\n\t"
+                    "v_cmp_eq_u32_e64 %[f2], %[w], %[y2]\n\t"
+                    "v_cmp_eq_u32_e64 %[e1], %[w], %[x1]\n\t"
+                    "v_cmp_eq_u32_e64 %[f1], %[w], %[y1]\n\t"
+                    "v_cmp_eq_u32_e64 %[e0], %[w], %[x0]\n\t"
+                    "v_cmp_eq_u32_e64 %[f0], %[w], %[y0]\n\t"
+                    "v_addc_co_u32_e64 %[ax], %[c], 0, 0, %[e3]\n\t"
+                    "v_addc_co_u32_e64 %[ay], %[c], 0, 0, %[f3]\n\t"
+                    "v_addc_co_u32_e64 %[ax], %[c], %[ax], %[ax], %[e2]\n\t"
+                    "v_addc_co_u32_e64 %[ay], %[c], %[ay], %[ay], %[f2]\n\t"
+                    "v_addc_co_u32_e64 %[ax], %[c], %[ax], %[ax], %[e1]\n\t"
+                    "v_addc_co_u32_e64 %[ay], %[c], %[ay], %[ay], %[f1]\n\t"
+                    "v_addc_co_u32_e64 %[ax], %[c], %[ax], %[ax], %[e0]\n\t"
+                    "v_addc_co_u32_e64 %[ay], %[c], %[ay], %[ay], %[f0]"
+                    : [ax] "=&v"(lo8), [ay] "=&v"(hi8), [e0] "=&s"(e0), [e1] "=&s"(e1), [e2] "=&s"(e2),
+                      [e3] "=&s"(e3), [f0] "=&s"(f0), [f1] "=&s"(f1), [f2] "=&s"(f2), [f3] "=&s"(f3),
+                      [c] "=&s"(carry)
+                    : [w] "v"(want), [x0] "v"(hq1.x), [x1] "v"(hq1.y), [x2] "v"(hq1.z), [x3] "v"(hq1.w),
+                      [y0] "v"(hq3.x), [y1] "v"(hq3.y), [y2] "v"(hq3.z), [y3] "v"(hq3.w));
                 asm("v_cmp_eq_u32_e64 %[e3], %[w], %[x3]\n\t"
                     "v_cmp_eq_u32_e64 %[f3], %[w], %[y3]\n\t"
                     "v_cmp_eq_u32_e64 %[e2], %[w], %[x2]\n\t"
@@ -571,16 +594,13 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                     "v_addc_co_u32_e64 %[ay], %[c], %[ay], %[ay], %[f1]\n\t"
                     "v_addc_co_u32_e64 %[ax], %[c], %[ax], %[ax], %[e0]\n\t"
                     "v_addc_co_u32_e64 %[ay], %[c], %[ay], %[ay], %[f0]"
-                    : [ax] "+v"(ax), [ay] "+v"(ay), [e0] "=&s"(e0), [e1] "=&s"(e1), [e2] "=&s"(e2),
+                    : [ax] "+v"(lo8), [ay] "+v"(hi8), [e0] "=&s"(e0), [e1] "=&s"(e1), [e2] "=&s"(e2),
                       [e3] "=&s"(e3), [f0] "=&s"(f0), [f1] "=&s"(f1), [f2] "=&s"(f2), [f3] "=&s"(f3),
                       [c] "=&s"(carry)
-                    : [w] "v"(want), [x0] "v"(x.x), [x1] "v"(x.y), [x2] "v"(x.z), [x3] "v"(x.w),
-                      [y0] "v"(y.x), [y1] "v"(y.y), [y2] "v"(y.z), [y3] "v"(y.w));
-            };
-            uint32_t m0 = 0, m1 = 0, m2 = 0, m3 = 0;  // four bits each, hashes 4k .. 4k+3
-            eight(hq0, hq1, m0, m1);
-            eight(hq2, hq3, m2, m3);
-            uint32_t m = (m0 | (m1 << 4)) | ((m2 | (m3 << 4)) << 8);
+                    : [w] "v"(want), [x0] "v"(hq0.x), [x1] "v"(hq0.y), [x2] "v"(hq0.z), [x3] "v"(hq0.w),
+                      [y0] "v"(hq2.x), [y1] "v"(hq2.y), [y2] "v"(hq2.z), [y3] "v"(hq2.w));
+            }
+            uint32_t m = lo8 | (hi8 << 8);
             m <<= 16 * h;
             {
                 // the two lanes of an element looked at 16 hashes each and join their masks
