@@ -648,6 +648,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             asm volatile("" : "+v"(claimed), "+v"(box0.x), "+v"(box0.y), "+v"(box1.x), "+v"(box1.y));
             // odd: a stay with several equal hashes, or a step claimed by two stays
             const uint32_t odd = (match & (match - 1)) | (claimed ^ mytag);
+            uint64_t stay_takes = mine_mask;  // lanes whose stay takes the score below
+            float cs_taken = cs_merged;
             if ((ballot(odd != 0u) & mine_mask) != 0 || (flags & 1)) {
                 // A stay with several equal hashes, or a step claimed by two stays (only
                 // possible after a CRC collision): replay the merges one by one in the
@@ -675,10 +677,14 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                     }
                 }
                 wave_fence();
-                if (h == 0) cs = sh.stay_score[i];
-                c0 = my_rec[0].step;
-                c1 = my_rec[1].step;
-            } else {
+                // the outcome takes the same way into the candidates as that of the usual route: every
+                // step's score as a mailbox entry of this time step, every even lane's stay as taken
+                box0 = make_uint2(now << 5, __float_as_uint(my_rec[0].step));
+                box1 = make_uint2(now << 5, __float_as_uint(my_rec[1].step));
+                cs_taken = sh.stay_score[i];
+                stay_takes = 0x5555555555555555ull;
+            }
+            {
                 // of every matched pair one side carries the folded score on, the other is dropped
                 // (the two compares first, the stay's own select between them and the selects that read
                 // their masks: two instructions lie between every compare and its reader)
@@ -694,7 +700,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                     : [c0] "+v"(c0), [c1] "+v"(c1), [cs] "+v"(cs), [t0] "=&v"(tag0), [t1] "=&v"(tag1),
                       [m0] "=&s"(hit0), [m1] "=&s"(hit1)
                     : [b0x] "v"(box0.x), [b1x] "v"(box1.x), [b0y] "v"(box0.y), [b1y] "v"(box1.y), [now] "s"(now),
-                      [csm] "v"(cs_merged), [mine] "s"(mine_mask));
+                      [csm] "v"(cs_taken), [mine] "s"(stay_takes));
             }
         }
 
