@@ -772,12 +772,27 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 slot1 = min(slot1, kW);
                 slots = min(slots, kW);
             }
-            sh.hash[slot0] = next.h0;
-            sh.elem[slot0] = Elem{next.h0, c0, next.info0, next.rest0};
-            sh.hash[slot1] = next.h1;
-            sh.elem[slot1] = Elem{next.h1, c1, next.info1, next.rest1};
-            sh.hash[slots] = hash;
-            sh.elem[slots] = Elem{hash, cs, next.infos, next.rests};
+            // The two addresses of a slot (its hash among the 32 contiguous hashes, its record) are
+            // formed by one shift-and-add each; derived from one another they cost a 64-bit multiply-add.
+            // A record goes out as two pairs of dwords, whose registers need not be neighbours.
+            typedef __attribute__((address_space(3))) uint32_t lds_u32;
+            const uint32_t hash_base = (uint32_t)(uintptr_t)(lds_u32 *)&sh.hash[0];
+            const uint32_t elem_base = (uint32_t)(uintptr_t)(lds_u32 *)&sh.elem[0].hash;
+            auto put = [&](int slot, uint32_t hsh, float sc, uint32_t inf, float rst) {
+                uint32_t at_hash, at_elem;
+                asm("v_lshl_add_u32 %0, %2, 2, %3\n\tv_lshl_add_u32 %1, %2, 4, %4"
+                    : "=&v"(at_hash), "=&v"(at_elem)
+                    : "v"(slot), "v"(hash_base), "v"(elem_base));
+                *(lds_u32 *)(uintptr_t)at_hash = hsh;
+                lds_u32 *rec = (lds_u32 *)(uintptr_t)at_elem;
+                rec[0] = hsh;
+                rec[1] = __float_as_uint(sc);
+                rec[2] = inf;
+                rec[3] = __float_as_uint(rst);
+            };
+            put(slot0, next.h0, c0, next.info0, next.rest0);
+            put(slot1, next.h1, c1, next.info1, next.rest1);
+            put(slots, hash, cs, next.infos, next.rests);
             wave_fence();
         }
         w = kept;
