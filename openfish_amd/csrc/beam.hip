@@ -19,8 +19,16 @@
 //
 // Stay/step merging: a stay of element i merges with the step (j, b_i) whose hash
 // crc(hash_j, b_i) equals hash_i.  The 2-bit CRC update is a bijection of the
-// 32-bit state, so this is the same as hash_j == crc^-1(hash_i, b_i): every lane
-// inverts its own hash once and compares it with the 32 previous hashes.
+// 32-bit state, so this is the same as hash_j == crc^-1(hash_i, b_i) =: want_i, the hash
+// of the element's sequence without its last base.  Every beam element carries both
+// words (a candidate's `want` is its parent's hash, or its parent's `want` for a stay), and
+// the element j is found through a hash index in LDS: every live element files
+// {hash, generation << 5 | slot} under some bits of its hash, reads its own entry back, and
+// looks up the entry filed under the same bits of `want`.  If every element finds its own
+// entry intact, all hashes are pairwise distinct and every existing partner is found by
+// exactly one probe (the full 32 bits are compared); otherwise (two elements in one
+// bucket, about one step in ten; equal hashes, only after a CRC collision) the step
+// falls back to comparing `want` with all 32 hashes.
 #include <hip/hip_runtime.h>
 
 #include <cfloat>
@@ -178,6 +186,34 @@ __device__ __forceinline__ int add_bit_of(int x, uint64_t mask) {
     return r;
 }
 __device__ __forceinline__ int popc64(uint64_t x) { return __builtin_popcountll(x); }
+// x + (float)h for the fp16 value h in the low half of a word, in one instruction: v_fma_mix_f32
+// converts the half operand on the fly and the product with 1.0 is exact, so the result is the
+// correctly rounded fp32 sum, bit for bit what a conversion followed by an addition gives
+__device__ __forceinline__ float add_half(uint32_t word, float x) {
+    float r;
+    asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(word), "v"(x));
+    return r;
+}
+// LDS accesses through a 32-bit LDS address
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#define LDS_AS __attribute__((address_space(3)))
+__device__ __forceinline__ f32x2 lds_load_f2(uint32_t at) { return *(const LDS_AS f32x2 *)(uintptr_t)at; }
+__device__ __forceinline__ u32x2 lds_load_u2(uint32_t at) { return *(const LDS_AS u32x2 *)(uintptr_t)at; }
+__device__ __forceinline__ float lds_load_f(uint32_t at) { return *(const LDS_AS float *)(uintptr_t)at; }
+__device__ __forceinline__ void lds_store_f2(uint32_t at, float a, float b) {
+    f32x2 v;
+    v.x = a;
+    v.y = b;
+    *(LDS_AS f32x2 *)(uintptr_t)at = v;
+}
+__device__ __forceinline__ void lds_store_f(uint32_t at, float a) { *(LDS_AS float *)(uintptr_t)at = a; }
+// (x & bits) | base in one instruction
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t bits, uint32_t base) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(bits), "v"(base));
+    return r;
+}
 
 __device__ __forceinline__ void wave_fence() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -298,25 +334,19 @@ struct BeamCfg {
 // one beam element as handed from one time step to the next
 struct __attribute__((aligned(16))) Elem {
     uint32_t hash;
-    float score;    // candidate score, guide term of its state included
+    uint32_t want;  // hash of the sequence without its last base: what a partner's hash has to equal
     uint32_t info;  // state | prev << 10 | stay << 15: the 16-bit slot the traceback reads
-    float rest;     // score minus that guide term: what the next time step starts from
-};
-// mailbox of one step candidate (index 4i+b): what a stay that merged with it leaves behind
-struct __attribute__((aligned(16))) SlotRec {
-    uint32_t tag;   // (t + 1) << 5 | stay element, written by the claiming stay at step t
-    float value;    // the step candidate's score after the merge
-    float step;     // the step candidate's own score (serial replay only)
-    uint32_t pad;
+    float rest;     // candidate score minus the guide term of its state: what the next time step starts from
+                    // (at the last time step: the candidate score itself, which picks the best survivor)
 };
 
 struct BeamShared {
-    uint32_t hash[kW + 4];  // hashes of the current beam, contiguous for the match sweep; entry kW
-    Elem elem[kW + 1];      // of both arrays is a dump slot for candidates that are not kept
-    SlotRec rec[4 * kW + 1];  // entry 4 * kW is a dump slot for lanes without a merge
-    float stay_score[kW];  // only used by the serial replay of merges
-    int ready;             // rows stored by the loader wave
-    int consumed;          // rows the search wave is done with
+    Elem elem[kW + 64];           // slots 0 .. kW-1; entry kW + lane is lane's dump slot for candidates that are not kept
+    float cand[4 * kW + 64];      // scores of the step candidates 4i+b while stays merge into them; then dump slots
+    float stay_score[kW];         // only used by the serial replay of merges
+    uint32_t claim[4 * kW + 64];  // only used when the hash index was not conclusive: who claimed step candidate 4j+b
+    int ready;                    // rows stored by the loader wave
+    int consumed;                 // rows the search wave is done with
 };
 
 // LDS of one chunk.  Score rows are kept as the caller lays them out: COLS = 4 transitions per
@@ -330,6 +360,12 @@ template <int S>
 struct BeamTrace {
     ofk_beam_slot_t slot[BeamCfg<S>::kTraceBlock][kW];
 };
+// Buckets of the hash index of one chunk (8 bytes each: hash, generation << 5 | slot).  With w
+// live elements two of them share a bucket in about w^2 / (2 * buckets) of the time steps.
+template <int S, int CPG>
+struct BeamIdx {
+    static constexpr int kBuckets = (S >= 1024 || CPG > 2) ? 2048 : 4096;
+};
 template <int S, int COLS>
 struct __attribute__((aligned(16))) BeamLds {
     // the ring is dead once the last time step has read its row; the traceback stages its blocks there
@@ -338,6 +374,15 @@ struct __attribute__((aligned(16))) BeamLds {
         BeamTrace<S> trace;
     };
     BeamShared sh;
+    uint2 idx_dump[64];  // where a dead lane files its leftovers instead of a bucket of the index
+};
+// All LDS of a workgroup, one object: the index tables come first and each is aligned to its
+// size, so that a bucket's address is (hash & bits) | table, one instruction.
+template <int S, int CPG, int COLS>
+struct __attribute__((aligned(BeamIdx<S, CPG>::kBuckets * 8))) BeamGroupLds {
+    uint2 idx[CPG][BeamIdx<S, CPG>::kBuckets];
+    BeamLds<S, COLS> chunk[CPG];
+    double lse[OFK_LSE_DOUBLES];  // coefficient table of the folds, one copy per workgroup
 };
 static_assert(sizeof(BeamTrace<64>) <= sizeof(BeamRing<64, 4>) && sizeof(BeamTrace<256>) <= sizeof(BeamRing<256, 4>) &&
                   sizeof(BeamTrace<1024>) <= sizeof(BeamRing<1024, 4>),
@@ -362,8 +407,9 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     constexpr int TB = Cfg::kTraceBlock;
 
     constexpr int kGroupChunks = CPG;
-    __shared__ BeamLds<S, COLS> lds[kGroupChunks];
-    __shared__ double lse[OFK_LSE_DOUBLES];  // coefficient table of the folds, one copy per workgroup
+    __shared__ BeamGroupLds<S, CPG, COLS> all;
+    auto &lds = all.chunk;
+    auto &lse = all.lse;
 
     // waves 0 .. kGroupChunks-1 search, the others load; wave k and wave k + kGroupChunks share a chunk
     const int wave = (int)(threadIdx.x >> 6);
@@ -383,6 +429,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         sh.consumed = 0;
     }
     for (int x = (int)threadIdx.x; x < OFK_LSE_DOUBLES; x += 128 * CPG) lse[x] = lse_table[x];
+    // the hash index starts empty: no entry may look like one of a real generation (tags start at 1 << 5)
+    for (int x = (int)threadIdx.x; x < kGroupChunks * BeamIdx<S, CPG>::kBuckets; x += 128 * CPG) (&all.idx[0][0])[x] = make_uint2(0u, 0u);
     __syncthreads();
     if (n >= N) return;  // odd batch: the last group has one chunk
 
@@ -434,6 +482,12 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     // ---- search wave ----
     const int i = lane >> 1;  // lanes 2i and 2i+1 hold element i; candidate order is lane order
     const int h = lane & 1;
+    constexpr int kBuckets = BeamIdx<S, CPG>::kBuckets;
+    constexpr uint32_t kBucketBits = (uint32_t)(kBuckets - 1) << 3;  // hash bits that address an 8-byte bucket
+    typedef __attribute__((address_space(3))) uint32_t lds_u32;
+    // LDS addresses of this chunk's index table (a multiple of its size) and of this lane's spare entry
+    const uint32_t idx_base = (uint32_t)(uintptr_t)(lds_u32 *)&all.idx[member][0].x;
+    const uint32_t idx_dump = (uint32_t)(uintptr_t)(lds_u32 *)&lds[member].idx_dump[lane].x;
 
     // seeding: the 32 best states of bwd[0] in ascending state order (src/beam_search.c:151-175)
     {
@@ -454,12 +508,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             if (wave_sum_i(c) >= kW) prefix = trial;
         }
         const float thr = key_float(prefix);
-        if (lane < kW) {
-            sh.hash[lane] = 0;
-            sh.elem[lane] = Elem{0u, 0.f, 0u, 0.f};
-        }
-        sh.rec[lane].tag = 0;  // tags of real time steps start at 1 << 5
-        sh.rec[lane + 64].tag = 0;
+        if (lane < kW) sh.elem[lane] = Elem{0u, 0u, 0u, 0.f};
         wave_fence();
         int taken = 0;
 #pragma unroll
@@ -471,20 +520,20 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 const uint32_t s = (uint32_t)(j * 64 + lane);
                 // flags bit 1 (tests): seeds that agree in their low four state bits share a hash
                 const uint32_t hs = crc32_word(kSeed, (flags & 2) ? (s & 15u) : s);
-                sh.hash[rank] = hs;
-                sh.elem[rank] = Elem{hs, 0.f, s, 0.f};
+                sh.elem[rank] = Elem{hs, crc2_inverse(hs, s & 3u), s, 0.f};
             }
             taken += popc64(m);
         }
         wave_fence();
     }
-    uint32_t hash, info;
+    uint32_t hash, want, info;
     float score;
     {
         const Elem e = sh.elem[i];
         hash = e.hash;
-        score = e.score;
+        want = e.want;
         info = e.info;
+        score = e.rest;
     }
     int state = (int)(info & 1023u);
     int w = kW;
@@ -502,58 +551,85 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     const uint32_t from = (uint32_t)i << 10, from_stay = from | (1u << 15);  // the element's index as "prev" of its candidates
     int rows_ready = 0;  // last value seen of the loader's counter; it is usually several rows ahead
     const int b0 = 2 * h;
+    const uint32_t cand_base = (uint32_t)(uintptr_t)(lds_u32 *)&sh.cand[0];
+    const uint32_t cand_mine = cand_base + 8u * (uint32_t)lane;           // candidates 4i+b0, 4i+b0+1
+    const uint32_t cand_dump = cand_base + 4u * (uint32_t)(4 * kW + lane);  // where a stay without a partner writes
     // What a time step reads from LDS depends only on the beam it starts from, so it is
     // fetched as soon as that beam is known (at the end of the previous step): the row
-    // entries of the lane's candidates and the 16 hashes this half of the wave compares with.
-    _Float16 r0h, r1h;
-    float2 g01;
+    // entries of the lane's candidates, and the hash index: the element's own entry goes in, is
+    // read back, and the entry filed under `want` is read.
+    uint32_t r0h, r1h;  // fp16 scores of the lane's two step candidates, each in the low half of a word
+    f32x2 g01;
     float gst;
-    uint4 hq0, hq1, hq2, hq3;
+    u32x2 probe;     // index entry found under `want`
+    uint32_t mine_back;  // tag found under the element's own hash
+    uint32_t tagv;   // generation << 5 | slot of this element (generation = time step + 1)
+    uint64_t vm = ~0ull;  // lanes of live elements
+    // ring addresses: the same in every lane, kept in scalar registers
+    const uint32_t ring_s = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(lds_u32 *)&row_s[0][0]);
+    const uint32_t ring_b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(lds_u32 *)&row_b[0][0]);
     auto fetch_row = [&](int tt) {
         while (rows_ready <= tt) {  // the counter is one LDS word: the same value in every lane
             rows_ready = __builtin_amdgcn_readfirstlane(observe(&sh.ready));
             if (rows_ready <= tt) __builtin_amdgcn_s_sleep(1);
         }
-        const int slot = tt % LR;
-        const _Float16 *rs = row_s[slot];
-        const float *rb = row_b[slot];
-        const int lo4 = (state << 2) & (S - 1);
-        const int top = state >> (BITS - 2);
-        r0h = rs[COLS * (lo4 + b0) + (COLS - 4) + top];
-        r1h = rs[COLS * (lo4 + b0 + 1) + (COLS - 4) + top];
-        g01 = *reinterpret_cast<const float2 *>(&rb[lo4 + b0]);
-        gst = rb[state];
-        const uint4 *hp = reinterpret_cast<const uint4 *>(&sh.hash[16 * h]);
-        hq0 = hp[0];
-        hq1 = hp[1];
-        hq2 = hp[2];
-        hq3 = hp[3];
+        const uint32_t slot = (uint32_t)tt % (uint32_t)LR;
+        const uint32_t rs = ring_s + slot * (uint32_t)(2 * COLS * S);  // scalar
+        const uint32_t rb = ring_b + slot * (uint32_t)(4 * S);
+        // scores of the candidates with bases b0, b0 + 1: rs[COLS * (lo4 + b0 + {0,1}) + (COLS - 4) + top];
+        // guide terms rb[lo4 + b0 + {0,1}] and rb[state]
+        const uint32_t st4 = (uint32_t)state << 2;
+        const uint32_t cand = and_or(st4, (uint32_t)(S - 1), (uint32_t)b0);  // lo4 + b0
+        const uint32_t top = ((uint32_t)state >> (BITS - 2)) << 1;  // byte offset of the dropped base's column
+        uint32_t at_s;
+        if constexpr (COLS == 4) at_s = (cand << 3) + rs;
+        else at_s = cand * 10u + rs;
+        at_s += top;
+        typedef __attribute__((address_space(3))) uint16_t lds_u16;
+        r0h = *(const lds_u16 *)(uintptr_t)(at_s + 2u * (COLS - 4));
+        r1h = *(const lds_u16 *)(uintptr_t)(at_s + 2u * (COLS - 4) + 2u * COLS);
+        g01 = lds_load_f2((cand << 2) + rb);
+        gst = lds_load_f(st4 + rb);
+        // hash index of the beam this step starts from; dead lanes file their leftovers apart
+        tagv = ((uint32_t)(tt + 1) << 5) | (uint32_t)i;
+        const uint32_t own = (uint32_t)pick_by_bit(vm, (int)and_or(hash, kBucketBits, idx_base), (int)idx_dump);
+        const uint32_t wanted = and_or(want, kBucketBits, idx_base);
+        lds_u32 *own_p = (lds_u32 *)(uintptr_t)own;
+        own_p[0] = hash;
+        own_p[1] = tagv;
+        wave_fence();  // one wave's LDS operations are carried out in order: the reads below see every lane's entry
+        probe = lds_load_u2(wanted);
+        mine_back = own_p[1];
     };
     fetch_row(0);
     for (int t = 0; t < T; ++t) {
-        const bool valid = i < w;
-        const uint64_t vm = ballot(valid);          // live elements, both halves
-        const uint64_t vs = vm & 0x5555555555555555ull;  // their stay candidates sit on the even lanes
-        const uint64_t odd_base = ballot((state & 1) != 0);  // lanes whose element ends in base 1 or 3
+        const uint64_t vs = vm & 0x5555555555555555ull;  // the stay candidates sit on the even lanes
         const int lo4 = (state << 2) & (S - 1);
-        const float r0 = (float)r0h;
-        const float r1 = (float)r1h;
-        float c0 = (score + r0) + g01.x;
-        float c1 = (score + r1) + g01.y;
+        // (score + transition) + guide, the CPU path's order of additions; the fp16 transition is
+        // converted inside the first addition
+        float c0 = add_half(r0h, score) + g01.x;
+        float c1 = add_half(r1h, score) + g01.y;
         float cs = (score + stay_h) + gst;
         publish(&sh.consumed, t + 1);  // everything this step needs of row t is in registers
-        SlotRec *my_rec = &sh.rec[4 * i + b0];
+        const uint32_t gen = (uint32_t)(t + 1) << 5;
 
-        // which previous element j has hash_j == crc^-1(hash_i, last base of i)
-        uint32_t match;
-        {
-            const uint32_t want = crc2_inverse(hash, (uint32_t)state & 3u);
-            // Bit k of m says whether hash k of this half equals `want`.  Each comparison is
-            // shifted into an accumulator with an add-with-carry (a = 2a + equal), two
-            // instructions per hash.  The low accumulator takes hashes 7..0, the high one hashes
-            // 15..8, eight comparisons at a time and the adds alternating between the two, so
-            // that no instruction waits for the one before it; each accumulator starts from the
-            // constant zero in its first add.
+        // which previous element j has hash_j == want_i: off the index if every live element found its
+        // own entry intact, else by comparing with every hash
+        uint32_t j;
+        uint64_t mine_mask;  // live even lanes whose stay has a partner
+        const uint64_t stale = ballot(mine_back != tagv) & vm;
+        if (stale == 0 && !(flags & 1)) {
+            const uint32_t d = probe.y - gen;  // below 32: an entry of this generation, and d is its slot
+            mine_mask = ballot(d < 32u) & ballot(probe.x == want) & vs;
+            j = d & 31u;
+        } else {
+            // Two live elements in one bucket (or with one hash).  Bit k of m says whether hash k of this
+            // half of the beam equals `want`: each comparison is shifted into an accumulator with an
+            // add-with-carry (a = 2a + equal), two accumulators so that no instruction waits for the one
+            // before it.
+            uint32_t hq[16];
+#pragma unroll
+            for (int k = 0; k < 16; ++k) hq[k] = sh.elem[16 * h + k].hash;
             uint32_t lo8, hi8;
             {
                 uint64_t e0, e1, e2, e3, f0, f1, f2, f3, carry;
@@ -576,8 +652,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                     : [ax] "=&v"(lo8), [ay] "=&v"(hi8), [e0] "=&s"(e0), [e1] "=&s"(e1), [e2] "=&s"(e2),
                       [e3] "=&s"(e3), [f0] "=&s"(f0), [f1] "=&s"(f1), [f2] "=&s"(f2), [f3] "=&s"(f3),
                       [c] "=&s"(carry)
-                    : [w] "v"(want), [x0] "v"(hq1.x), [x1] "v"(hq1.y), [x2] "v"(hq1.z), [x3] "v"(hq1.w),
-                      [y0] "v"(hq3.x), [y1] "v"(hq3.y), [y2] "v"(hq3.z), [y3] "v"(hq3.w));
+                    : [w] "v"(want), [x0] "v"(hq[4]), [x1] "v"(hq[5]), [x2] "v"(hq[6]), [x3] "v"(hq[7]),
+                      [y0] "v"(hq[12]), [y1] "v"(hq[13]), [y2] "v"(hq[14]), [y3] "v"(hq[15]));
                 asm("v_cmp_eq_u32_e64 %[e3], %[w], %[x3]\n\t"
                     "v_cmp_eq_u32_e64 %[f3], %[w], %[y3]\n\t"
                     "v_cmp_eq_u32_e64 %[e2], %[w], %[x2]\n\t"
@@ -597,111 +673,84 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                     : [ax] "+v"(lo8), [ay] "+v"(hi8), [e0] "=&s"(e0), [e1] "=&s"(e1), [e2] "=&s"(e2),
                       [e3] "=&s"(e3), [f0] "=&s"(f0), [f1] "=&s"(f1), [f2] "=&s"(f2), [f3] "=&s"(f3),
                       [c] "=&s"(carry)
-                    : [w] "v"(want), [x0] "v"(hq0.x), [x1] "v"(hq0.y), [x2] "v"(hq0.z), [x3] "v"(hq0.w),
-                      [y0] "v"(hq2.x), [y1] "v"(hq2.y), [y2] "v"(hq2.z), [y3] "v"(hq2.w));
+                    : [w] "v"(want), [x0] "v"(hq[0]), [x1] "v"(hq[1]), [x2] "v"(hq[2]), [x3] "v"(hq[3]),
+                      [y0] "v"(hq[8]), [y1] "v"(hq[9]), [y2] "v"(hq[10]), [y3] "v"(hq[11]));
             }
             uint32_t m = lo8 | (hi8 << 8);
             m <<= 16 * h;
-            {
-                // the two lanes of an element looked at 16 hashes each and join their masks
-                m |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1 /* quad_perm:[1,0,3,2] */, 0xF, 0xF, true);
-            }
+            // the two lanes of an element looked at 16 hashes each and join their masks
+            m |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1 /* quad_perm:[1,0,3,2] */, 0xF, 0xF, true);
             const uint32_t live = w >= 32 ? 0xFFFFFFFFu : ((1u << w) - 1u);
-            match = m & live;  // of a dead lane: leftovers, masked out below
-        }
-
-        // merge stays with the step spelling the same sequence (src/beam_search.c:281-316).
-        // The stay's lane fetches the step's score from the lane that holds it, folds the two,
-        // keeps its half of the outcome and leaves the step's half in the step's mailbox.
-        // Conditions that hold per lane are kept as wave-wide masks in scalar registers and combined
-        // there; a select then takes its mask as it is.  (A condition put together from vector
-        // instructions right before its use costs the wait states between a compare and its reader,
-        // and a wave that is alone on its SIMD pays a whole issue slot for each.)
-        const uint64_t mine_mask = ballot(match != 0u) & vs;  // live even lanes whose stay has a partner
-        if (mine_mask != 0) {
-            const uint32_t now = (uint32_t)(t + 1);
-            const uint32_t mytag = (now << 5) | (uint32_t)i;
-            const int j = __builtin_ctz(match | 0x80000000u) & 31;
-            const int bi = state & 3;
-            const int holder = (2 * j + (bi >> 1)) << 2;  // the lane with element j and base bi, as a byte index
-            const float o0 = __int_as_float(__builtin_amdgcn_ds_bpermute(holder, __float_as_int(c0)));
-            const float o1 = __int_as_float(__builtin_amdgcn_ds_bpermute(holder, __float_as_int(c1)));
-            const float other = __int_as_float(pick_by_bit(odd_base, __float_as_int(o1), __float_as_int(o0)));
-            const uint64_t stay_wins = ballot(cs > other);
-            // every lane goes through the fold and the mailbox, lanes without a merge with whatever
-            // their registers hold and the dump slot as target: no exec masking on the way
-            // the fold from hardware exp/log where that provably rounds like the CPU path's double
-            // arithmetic (all but a few merges in a thousand at usual score magnitudes)
-            bool settled;
-            float folded = log_sum_exp_estimate(cs, other, settled);
-            if ((ballot(!settled) & mine_mask) != 0) folded = log_sum_exp(cs, other, lse);
-            const int target = pick_by_bit(mine_mask, 4 * j + bi, 4 * kW);
-            const float cs_merged = __int_as_float(pick_by_bit(stay_wins, __float_as_int(folded), __float_as_int(-FLT_MAX)));
-            *reinterpret_cast<uint2 *>(&sh.rec[target]) = make_uint2(
-                mytag, (uint32_t)pick_by_bit(stay_wins, __float_as_int(-FLT_MAX), __float_as_int(folded)));
+            const uint32_t match = m & live;
+            mine_mask = ballot(match != 0u) & vs;
+            j = (uint32_t)__builtin_ctz(match | 0x80000000u) & 31u;
+            // Merges in parallel need every stay to have one partner and every step candidate one claimant.
+            // Otherwise (only possible after a CRC collision; flags bit 0 forces it) the merges are
+            // replayed one by one in the CPU path's order, from the scores as they were before any merge.
+            const uint32_t claim_at = (uint32_t)pick_by_bit(mine_mask, (int)(4u * j + ((uint32_t)state & 3u)), 4 * kW + lane);
+            sh.claim[claim_at] = (uint32_t)i;
             wave_fence();
-            uint32_t claimed = sh.rec[target].tag;
-            uint2 box0 = *reinterpret_cast<const uint2 *>(&my_rec[0]);
-            uint2 box1 = *reinterpret_cast<const uint2 *>(&my_rec[1]);
-            // keep the three reads together in one LDS round trip (the compiler would otherwise
-            // sink the mailbox reads below the branch that follows)
-            asm volatile("" : "+v"(claimed), "+v"(box0.x), "+v"(box0.y), "+v"(box1.x), "+v"(box1.y));
-            // odd: a stay with several equal hashes, or a step claimed by two stays
-            const uint32_t odd = (match & (match - 1)) | (claimed ^ mytag);
-            uint64_t stay_takes = mine_mask;  // lanes whose stay takes the score below
-            float cs_taken = cs_merged;
+            const uint32_t claimed = sh.claim[claim_at];
+            const uint32_t odd = (match & (match - 1u)) | (claimed ^ (uint32_t)i);
             if ((ballot(odd != 0u) & mine_mask) != 0 || (flags & 1)) {
-                // A stay with several equal hashes, or a step claimed by two stays (only
-                // possible after a CRC collision): replay the merges one by one in the
-                // CPU path's order, from the scores as they were before any merge.
-                my_rec[0].step = c0;
-                my_rec[1].step = c1;
+                lds_store_f2(cand_mine, c0, c1);
                 if (h == 0) sh.stay_score[i] = cs;
                 wave_fence();
                 if (lane == 0) {
                     for (int a = 0; a < w; ++a) {
-                        const uint32_t ha = sh.hash[a];
+                        const uint32_t ha = sh.elem[a].hash;
                         const uint32_t base = sh.elem[a].info & 3u;
                         for (int b = 0; b < w; ++b) {
-                            if (crc2(sh.hash[b], base) != ha) continue;
-                            SlotRec *st = &sh.rec[4 * b + (int)base];
-                            const float both = log_sum_exp(sh.stay_score[a], st->step, lse);
-                            if (sh.stay_score[a] > st->step) {
+                            if (crc2(sh.elem[b].hash, base) != ha) continue;
+                            float *st = &sh.cand[4 * b + (int)base];
+                            const float both = log_sum_exp(sh.stay_score[a], *st, lse);
+                            if (sh.stay_score[a] > *st) {
                                 sh.stay_score[a] = both;
-                                st->step = -FLT_MAX;
+                                *st = -FLT_MAX;
                             } else {
-                                st->step = both;
+                                *st = both;
                                 sh.stay_score[a] = -FLT_MAX;
                             }
                         }
                     }
                 }
                 wave_fence();
-                // the outcome takes the same way into the candidates as that of the usual route: every
-                // step's score as a mailbox entry of this time step, every even lane's stay as taken
-                box0 = make_uint2(now << 5, __float_as_uint(my_rec[0].step));
-                box1 = make_uint2(now << 5, __float_as_uint(my_rec[1].step));
-                cs_taken = sh.stay_score[i];
-                stay_takes = 0x5555555555555555ull;
+                const f32x2 c01 = lds_load_f2(cand_mine);
+                c0 = c01.x;
+                c1 = c01.y;
+                if (h == 0) cs = sh.stay_score[i];
+                mine_mask = 0;
             }
-            {
-                // of every matched pair one side carries the folded score on, the other is dropped
-                // (the two compares first, the stay's own select between them and the selects that read
-                // their masks: two instructions lie between every compare and its reader)
-                uint32_t tag0, tag1;
-                uint64_t hit0, hit1;
-                asm("v_lshrrev_b32 %[t0], 5, %[b0x]\n\t"
-                    "v_lshrrev_b32 %[t1], 5, %[b1x]\n\t"
-                    "v_cmp_eq_u32_e64 %[m0], %[now], %[t0]\n\t"
-                    "v_cmp_eq_u32_e64 %[m1], %[now], %[t1]\n\t"
-                    "v_cndmask_b32_e64 %[cs], %[cs], %[csm], %[mine]\n\t"
-                    "v_cndmask_b32_e64 %[c0], %[c0], %[b0y], %[m0]\n\t"
-                    "v_cndmask_b32_e64 %[c1], %[c1], %[b1y], %[m1]"
-                    : [c0] "+v"(c0), [c1] "+v"(c1), [cs] "+v"(cs), [t0] "=&v"(tag0), [t1] "=&v"(tag1),
-                      [m0] "=&s"(hit0), [m1] "=&s"(hit1)
-                    : [b0x] "v"(box0.x), [b1x] "v"(box1.x), [b0y] "v"(box0.y), [b1y] "v"(box1.y), [now] "s"(now),
-                      [csm] "v"(cs_taken), [mine] "s"(stay_takes));
-            }
+        }
+
+        // merge stays with the step spelling the same sequence (src/beam_search.c:281-316).  Every lane
+        // files its two step candidates; a stay with a partner reads the partner's score, folds the
+        // two, keeps its half of the outcome and overwrites the partner with the other half; every
+        // lane reads its step candidates back.  Lanes without a merge go through the same
+        // instructions with whatever their registers hold and a dump slot as target: no exec
+        // masking on the way.  Conditions are kept as wave-wide masks in scalar registers and combined
+        // there; a select takes its mask as it is.
+        if (mine_mask != 0) {
+            lds_store_f2(cand_mine, c0, c1);
+            uint32_t at;  // the partner: step candidate 4j + last base of this element
+            asm("v_lshl_add_u32 %0, %1, 4, %2" : "=v"(at) : "v"(j), "v"(cand_base + (((uint32_t)state & 3u) << 2)));
+            wave_fence();
+            const float other = lds_load_f(at);
+            const uint64_t stay_wins = ballot(cs > other) & mine_mask;
+            const uint64_t step_wins = mine_mask & ~stay_wins;
+            // the fold from hardware exp/log where that provably rounds like the CPU path's double
+            // arithmetic (all but a few merges in a thousand at usual score magnitudes)
+            bool settled;
+            float folded = log_sum_exp_estimate(cs, other, settled);
+            if ((ballot(!settled) & mine_mask) != 0) folded = log_sum_exp(cs, other, lse);
+            const uint32_t target = (uint32_t)pick_by_bit(mine_mask, (int)at, (int)cand_dump);
+            lds_store_f(target, __int_as_float(pick_by_bit(step_wins, __float_as_int(folded), __float_as_int(-FLT_MAX))));
+            cs = __int_as_float(pick_by_bit(stay_wins, __float_as_int(folded), __float_as_int(cs)));
+            cs = __int_as_float(pick_by_bit(step_wins, __float_as_int(-FLT_MAX), __float_as_int(cs)));
+            wave_fence();
+            const f32x2 c01 = lds_load_f2(cand_mine);
+            c0 = c01.x;
+            c1 = c01.y;
         }
 
         // cut-off (src/beam_search.c:320-381)
@@ -749,6 +798,10 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
 
         // survivors in candidate order: steps (i, b) by i then b, then stays by i
         {
+            // The masks may come straight from vector compares; the selects below are written as
+            // instructions and read them as scalar operands, which a vector instruction may do only two
+            // instructions after a vector instruction wrote them: scalar copies are safe to read at once.
+            asm volatile("s_mov_b64 %0, %0\n\ts_mov_b64 %1, %1\n\ts_mov_b64 %2, %2" : "+s"(k0), "+s"(k1), "+s"(ks));
             // kept candidates on lower lanes: masked bit counts
             auto lower = [&](uint64_t mask, int start) {
                 return (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
@@ -759,52 +812,55 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             const int rank0 = lower(k1, lower(k0, 0));
             const int rank1 = add_bit_of(rank0, k0);
             const int ranks = lower(ks, popc64(k0) + popc64(k1));
-            // every lane stores all three of its candidates, the ones that are dropped into the dump
+            // every lane stores all three of its candidates, the ones that are dropped into its own dump
             // slot: no exec masking on the path from the cut-off to the next beam.  Kept candidates
             // beyond the width exist only after the ten-guess exit of the bisection; a branch that is
             // almost never taken sends them to the dump slot as well.
-            int slot0 = pick_by_bit(k0, rank0, kW);
-            int slot1 = pick_by_bit(k1, rank1, kW);
-            int slots = pick_by_bit(ks, ranks, kW);
+            const int dump = kW + lane;
+            int slot0 = pick_by_bit(k0, rank0, dump);
+            int slot1 = pick_by_bit(k1, rank1, dump);
+            int slots = pick_by_bit(ks, ranks, dump);
             if (overfull) {
                 asm volatile("");  // keeps this a branch instead of three selects on every step
-                slot0 = min(slot0, kW);
-                slot1 = min(slot1, kW);
-                slots = min(slots, kW);
+                slot0 = slot0 >= kW ? dump : slot0;
+                slot1 = slot1 >= kW ? dump : slot1;
+                slots = slots >= kW ? dump : slots;
             }
-            // The two addresses of a slot (its hash among the 32 contiguous hashes, its record) are
-            // formed by one shift-and-add each; derived from one another they cost a 64-bit multiply-add.
-            // A record goes out as two pairs of dwords, whose registers need not be neighbours.
-            typedef __attribute__((address_space(3))) uint32_t lds_u32;
-            const uint32_t hash_base = (uint32_t)(uintptr_t)(lds_u32 *)&sh.hash[0];
+            if (t == T - 1) {
+                // the last beam is ranked by its candidate scores (src/beam_search.c:398-414)
+                asm volatile("");  // a branch taken once, not three selects in every step
+                next.rest0 = c0;
+                next.rest1 = c1;
+                next.rests = cs;
+            }
             const uint32_t elem_base = (uint32_t)(uintptr_t)(lds_u32 *)&sh.elem[0].hash;
-            auto put = [&](int slot, uint32_t hsh, float sc, uint32_t inf, float rst) {
-                uint32_t at_hash, at_elem;
-                asm("v_lshl_add_u32 %0, %2, 2, %3\n\tv_lshl_add_u32 %1, %2, 4, %4"
-                    : "=&v"(at_hash), "=&v"(at_elem)
-                    : "v"(slot), "v"(hash_base), "v"(elem_base));
-                *(lds_u32 *)(uintptr_t)at_hash = hsh;
-                lds_u32 *rec = (lds_u32 *)(uintptr_t)at_elem;
-                rec[0] = hsh;
-                rec[1] = __float_as_uint(sc);
-                rec[2] = inf;
-                rec[3] = __float_as_uint(rst);
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            auto put = [&](int slot, uint32_t hsh, uint32_t wnt, uint32_t inf, float rst) {
+                uint32_t at_elem;
+                asm("v_lshl_add_u32 %0, %1, 4, %2" : "=v"(at_elem) : "v"(slot), "v"(elem_base));
+                u32x4 rec;
+                rec.x = hsh;
+                rec.y = wnt;
+                rec.z = inf;
+                rec.w = __float_as_uint(rst);
+                *(__attribute__((address_space(3))) u32x4 *)(uintptr_t)at_elem = rec;
             };
-            put(slot0, next.h0, c0, next.info0, next.rest0);
-            put(slot1, next.h1, c1, next.info1, next.rest1);
-            put(slots, hash, cs, next.infos, next.rests);
+            put(slot0, next.h0, hash, next.info0, next.rest0);
+            put(slot1, next.h1, hash, next.info1, next.rest1);
+            put(slots, hash, want, next.infos, next.rests);
             wave_fence();
         }
         w = kept;
-        // every lane reads its slot; slots past the new width hold leftovers and are masked here
-        float rest;
+        vm = w > 0 ? ~0ull >> (64 - 2 * w) : 0ull;  // (the best candidate is always kept: w is zero only after NaN scores)
+        // every lane reads its slot; slots past the new width hold leftovers: they count as dead through
+        // their score and persist as zero, which is what the CPU path's untouched slots hold (a beam
+        // cut below 1 empties the beam, and the traceback then walks such slots)
         {
             const Elem e = sh.elem[i];
-            const bool in = i < w;
             hash = e.hash;
-            score = in ? e.score : -FLT_MAX;
-            info = in ? e.info : 0u;
-            rest = in ? e.rest : -FLT_MAX;
+            want = e.want;
+            info = (uint32_t)pick_by_bit(vm, (int)e.info, 0);
+            score = __int_as_float(pick_by_bit(vm, __float_as_int(e.rest), __float_as_int(-FLT_MAX)));
         }
         state = (int)(info & 1023u);
         if (t + 1 < T) fetch_row(t + 1);
@@ -812,27 +868,21 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // last block: the best survivor goes to slot 0 (src/beam_search.c:398-414)
         if (t == T - 1) {
             const bool in = i < w;
-            const float top_score = wave_max(in ? score : -FLT_MAX);
+            const float top_score = wave_max(score);
             const uint64_t at = ballot(in && h == 0 && score == top_score);
             const int arg_lane = (top_score > -FLT_MAX && at != 0) ? __builtin_ctzll(at) : 0;  // an even lane
             const int arg = arg_lane >> 1;
             if (arg != 0) {
-                const uint32_t hash0 = lane_u(hash, 0), hasha = lane_u(hash, arg_lane);
                 const uint32_t in0 = lane_u(info, 0), ina = lane_u(info, arg_lane);
-                const float re0 = lane_f(rest, 0), rea = lane_f(rest, arg_lane);
-                if (i == 0) { hash = hasha; info = ina; rest = rea; }
-                if (i == arg) { hash = hash0; info = in0; rest = re0; }
-                state = (int)(info & 1023u);
+                if (i == 0) info = ina;
+                if (i == arg) info = in0;
             }
         }
 
-        // drop the guide term again and persist the slot (src/beam_search.c:417-427); the
-        // difference was taken by the lane that held the candidate, which had the term at hand
-        score = rest;
-        // both halves hold the same element and store the same slot; slots past the width are never
-        // followed by the traceback
-        bv[(size_t)(t + 1) * kW + i] =
-            (ofk_beam_slot_t)info;
+        // persist the slot (src/beam_search.c:417-427); the guide term was dropped again by the lane
+        // that held the candidate, which had the term at hand.  Both halves hold the same element
+        // and store the same slot; slots past the width are never followed by the traceback
+        bv[(size_t)(t + 1) * kW + i] = (ofk_beam_slot_t)info;
     }
 
     // ---- traceback from slot 0 of the last block (src/beam_search.c:432-439) ----
