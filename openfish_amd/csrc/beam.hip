@@ -33,6 +33,7 @@
 
 #include <cfloat>
 #include <mutex>
+#include <type_traits>
 
 #include "kernels.h"
 
@@ -327,17 +328,16 @@ struct BeamCfg {
     static constexpr int kBits = S == 64 ? 6 : S == 256 ? 8 : 10;
     static constexpr int kLdsRows = S >= 1024 ? 3 : S >= 256 ? 4 : 6;  // LDS ring depth
     static constexpr int kRegRows = S >= 1024 ? 3 : 6;  // rows in flight in registers (3 or 6)
-    // time steps staged per traceback block; the staging buffers reuse the memory of the ring
-    static constexpr int kTraceBlock = S >= 256 ? 128 : 64;
 };
 
-// one beam element as handed from one time step to the next
+// one beam element as handed from one time step to the next: three words of a 16-byte slot, written
+// by one 96-bit store (an LDS store costs by its width, whatever the number of enabled lanes)
 struct __attribute__((aligned(16))) Elem {
     uint32_t hash;
-    uint32_t want;  // hash of the sequence without its last base: what a partner's hash has to equal
-    uint32_t info;  // state | prev << 10 | stay << 15: the 16-bit slot the traceback reads
     float rest;     // candidate score minus the guide term of its state: what the next time step starts from
                     // (at the last time step: the candidate score itself, which picks the best survivor)
+    uint32_t info;  // state | prev << 10 | stay << 15: the 16-bit slot the traceback reads
+    uint32_t pad;
 };
 
 struct BeamShared {
@@ -356,10 +356,6 @@ struct BeamRing {
     _Float16 row_s[BeamCfg<S>::kLdsRows][COLS * S];
     float row_b[BeamCfg<S>::kLdsRows][S];
 };
-template <int S>
-struct BeamTrace {
-    ofk_beam_slot_t slot[BeamCfg<S>::kTraceBlock][kW];
-};
 // Buckets of the hash index of one chunk (8 bytes each: hash, generation << 5 | slot).  With w
 // live elements two of them share a bucket in about w^2 / (2 * buckets) of the time steps.
 template <int S, int CPG>
@@ -368,11 +364,7 @@ struct BeamIdx {
 };
 template <int S, int COLS>
 struct __attribute__((aligned(16))) BeamLds {
-    // the ring is dead once the last time step has read its row; the traceback stages its blocks there
-    union {
-        BeamRing<S, COLS> ring;
-        BeamTrace<S> trace;
-    };
+    BeamRing<S, COLS> ring;
     BeamShared sh;
     uint2 idx_dump[64];  // where a dead lane files its leftovers instead of a bucket of the index
 };
@@ -384,9 +376,7 @@ struct __attribute__((aligned(BeamIdx<S, CPG>::kBuckets * 8))) BeamGroupLds {
     BeamLds<S, COLS> chunk[CPG];
     double lse[OFK_LSE_DOUBLES];  // coefficient table of the folds, one copy per workgroup
 };
-static_assert(sizeof(BeamTrace<64>) <= sizeof(BeamRing<64, 4>) && sizeof(BeamTrace<256>) <= sizeof(BeamRing<256, 4>) &&
-                  sizeof(BeamTrace<1024>) <= sizeof(BeamRing<1024, 4>),
-              "traceback staging must fit into the ring");
+
 
 // CPG chunks per workgroup.  The waves of a group are dealt round over the four SIMDs of
 // its compute unit (wave k and wave k + 4 share one), while two-wave groups were measured
@@ -404,7 +394,6 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     constexpr int BITS = Cfg::kBits;
     constexpr int LR = Cfg::kLdsRows;
     constexpr int RR = Cfg::kRegRows;
-    constexpr int TB = Cfg::kTraceBlock;
 
     constexpr int kGroupChunks = CPG;
     __shared__ BeamGroupLds<S, CPG, COLS> all;
@@ -419,7 +408,6 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     auto &row_s = lds[member].ring.row_s;
     auto &row_b = lds[member].ring.row_b;
     BeamShared &sh = lds[member].sh;
-    auto &trace = lds[member].trace.slot;
     const size_t row_stride = (size_t)N * COLS * S;
     const _Float16 *sc_n = scores + (size_t)n * COLS * S;
     const float *bw_n = bwd + (size_t)n * (size_t)(T + 1) * S;
@@ -508,7 +496,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             if (wave_sum_i(c) >= kW) prefix = trial;
         }
         const float thr = key_float(prefix);
-        if (lane < kW) sh.elem[lane] = Elem{0u, 0u, 0u, 0.f};
+        if (lane < kW) sh.elem[lane] = Elem{0u, 0.f, 0u, 0u};
         wave_fence();
         int taken = 0;
 #pragma unroll
@@ -520,22 +508,22 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 const uint32_t s = (uint32_t)(j * 64 + lane);
                 // flags bit 1 (tests): seeds that agree in their low four state bits share a hash
                 const uint32_t hs = crc32_word(kSeed, (flags & 2) ? (s & 15u) : s);
-                sh.elem[rank] = Elem{hs, crc2_inverse(hs, s & 3u), s, 0.f};
+                sh.elem[rank] = Elem{hs, 0.f, s, 0u};
             }
             taken += popc64(m);
         }
         wave_fence();
     }
-    uint32_t hash, want, info;
+    uint32_t hash, want, info;  // want: the hash of the sequence without its last base, what a partner's hash has to equal
     float score;
     {
         const Elem e = sh.elem[i];
         hash = e.hash;
-        want = e.want;
         info = e.info;
         score = e.rest;
     }
     int state = (int)(info & 1023u);
+    want = crc2_inverse(hash, (uint32_t)state & 3u);
     int w = kW;
     ofk_beam_slot_t *bv = beam + (size_t)n * (size_t)(T + 1) * kW;
     bv[i] = (ofk_beam_slot_t)state;
@@ -569,7 +557,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
     const uint32_t ring_s = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(lds_u32 *)&row_s[0][0]);
     const uint32_t ring_b = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(lds_u32 *)&row_b[0][0]);
     auto fetch_row = [&](int tt) {
-        while (rows_ready <= tt) {  // the counter is one LDS word: the same value in every lane
+        while (__builtin_expect(rows_ready <= tt, 0)) {  // the counter is one LDS word: the same value in every lane
             rows_ready = __builtin_amdgcn_readfirstlane(observe(&sh.ready));
             if (rows_ready <= tt) __builtin_amdgcn_s_sleep(1);
         }
@@ -602,7 +590,12 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         mine_back = own_p[1];
     };
     fetch_row(0);
-    for (int t = 0; t < T; ++t) {
+    const uint64_t replay_all = (flags & 1) ? ~0ull : 0ull;
+    // One time step.  The last one (LAST) differs in what it hands on (nothing is fetched for a next
+    // step, the best survivor goes to slot 0) and is compiled apart, so that the others carry no
+    // test for it.
+    auto step = [&](const int t, auto last_tag) {
+        constexpr bool LAST = decltype(last_tag)::value;
         const uint64_t vs = vm & 0x5555555555555555ull;  // the stay candidates sit on the even lanes
         const int lo4 = (state << 2) & (S - 1);
         // (score + transition) + guide, the CPU path's order of additions; the fp16 transition is
@@ -617,8 +610,8 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // own entry intact, else by comparing with every hash
         uint32_t j;
         uint64_t mine_mask;  // live even lanes whose stay has a partner
-        const uint64_t stale = ballot(mine_back != tagv) & vm;
-        if (stale == 0 && !(flags & 1)) {
+        const uint64_t stale = (ballot(mine_back != tagv) & vm) | replay_all;
+        if (__builtin_expect(stale == 0, 1)) {
             const uint32_t d = probe.y - gen;  // below 32: an entry of this generation, and d is its slot
             mine_mask = ballot(d < 32u) & ballot(probe.x == want) & vs;
             j = d & 31u;
@@ -730,7 +723,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // instructions with whatever their registers hold and a dump slot as target: no exec
         // masking on the way.  Conditions are kept as wave-wide masks in scalar registers and combined
         // there; a select takes its mask as it is.
-        if (mine_mask != 0) {
+        if (__builtin_expect(mine_mask != 0, 1)) {
             lds_store_f2(cand_mine, c0, c1);
             uint32_t at;  // the partner: step candidate 4j + last base of this element
             asm("v_lshl_add_u32 %0, %1, 4, %2" : "=v"(at) : "v"(j), "v"(cand_base + (((uint32_t)state & 3u) << 2)));
@@ -742,7 +735,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             // arithmetic (all but a few merges in a thousand at usual score magnitudes)
             bool settled;
             float folded = log_sum_exp_estimate(cs, other, settled);
-            if ((ballot(!settled) & mine_mask) != 0) folded = log_sum_exp(cs, other, lse);
+            if (__builtin_expect((ballot(!settled) & mine_mask) != 0, 0)) folded = log_sum_exp(cs, other, lse);
             const uint32_t target = (uint32_t)pick_by_bit(mine_mask, (int)at, (int)cand_dump);
             lds_store_f(target, __int_as_float(pick_by_bit(step_wins, __float_as_int(folded), __float_as_int(-FLT_MAX))));
             cs = __int_as_float(pick_by_bit(stay_wins, __float_as_int(folded), __float_as_int(cs)));
@@ -764,14 +757,15 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         uint64_t k0 = ballot(c0 >= cut) & vm, k1 = ballot(c1 >= cut) & vm, ks = ballot(cs >= cut) & vs;
         int kept = popc64(k0) + popc64(k1) + popc64(ks);
         bool overfull = false;  // more candidates than the width pass the final cut (the same in every lane)
-        if (kept > kW) {
+        if (__builtin_expect(kept > kW, 1)) {
             // Bisection between the cut and the best score.  Every cut tried in here lies above
             // (-FLT_MAX + best) / 2, so dead lanes and dropped candidates never pass and the
             // ballots need no mask.  (lo + hi) / 2 is the CPU path's (cut + hi) / 2 or
             // (cut + lo) / 2: one of the two bounds is the cut just tried.
             float lo = cut, hi = best;
-            int guesses = 1;
-            for (;;) {
+            bool found = false;
+#pragma unroll
+            for (int guess = 2; guess < 10; ++guess) {
                 const bool up = kept > kW;
                 lo = up ? cut : lo;
                 hi = up ? hi : cut;
@@ -780,20 +774,23 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 k1 = ballot(c1 >= cut);
                 ks = ballot(cs >= cut);
                 kept = popc64(k0) + popc64(k1) + popc64(ks);
-                ++guesses;
-                if ((unsigned)(kept - (kW * 8) / 10) <= (unsigned)(kW - (kW * 8) / 10)) break;  // 25..32 kept
-                asm volatile("");  // two scalar branches, not one condition put together from lane masks
-                if (guesses >= 10) break;
+                if ((unsigned)(kept - (kW * 8) / 10) <= (unsigned)(kW - (kW * 8) / 10)) {  // 25..32 kept
+                    found = true;
+                    break;
+                }
             }
-            if (guesses == 10) {
+            if (__builtin_expect(!found, 0)) {
+                // The tenth guess: the CPU path moves its bounds once more, tries a cut whose count it
+                // never looks at, and settles for the upper bound, whatever that keeps.
+                hi = kept > kW ? hi : cut;
                 cut = hi;
                 k0 = ballot(c0 >= cut);
                 k1 = ballot(c1 >= cut);
                 ks = ballot(cs >= cut);
                 kept = popc64(k0) + popc64(k1) + popc64(ks);
+                overfull = kept > kW;
+                if (overfull) kept = kW;
             }
-            overfull = kept > kW;
-            if (overfull) kept = kW;
         }
 
         // survivors in candidate order: steps (i, b) by i then b, then stays by i
@@ -820,34 +817,32 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
             int slot0 = pick_by_bit(k0, rank0, dump);
             int slot1 = pick_by_bit(k1, rank1, dump);
             int slots = pick_by_bit(ks, ranks, dump);
-            if (overfull) {
+            if (__builtin_expect(overfull, 0)) {
                 asm volatile("");  // keeps this a branch instead of three selects on every step
                 slot0 = slot0 >= kW ? dump : slot0;
                 slot1 = slot1 >= kW ? dump : slot1;
                 slots = slots >= kW ? dump : slots;
             }
-            if (t == T - 1) {
+            if constexpr (LAST) {
                 // the last beam is ranked by its candidate scores (src/beam_search.c:398-414)
-                asm volatile("");  // a branch taken once, not three selects in every step
                 next.rest0 = c0;
                 next.rest1 = c1;
                 next.rests = cs;
             }
             const uint32_t elem_base = (uint32_t)(uintptr_t)(lds_u32 *)&sh.elem[0].hash;
-            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-            auto put = [&](int slot, uint32_t hsh, uint32_t wnt, uint32_t inf, float rst) {
+            typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+            auto put = [&](int slot, uint32_t hsh, uint32_t inf, float rst) {
                 uint32_t at_elem;
                 asm("v_lshl_add_u32 %0, %1, 4, %2" : "=v"(at_elem) : "v"(slot), "v"(elem_base));
-                u32x4 rec;
+                u32x3 rec;
                 rec.x = hsh;
-                rec.y = wnt;
+                rec.y = __float_as_uint(rst);
                 rec.z = inf;
-                rec.w = __float_as_uint(rst);
-                *(__attribute__((address_space(3))) u32x4 *)(uintptr_t)at_elem = rec;
+                *(LDS_AS u32x3 *)(uintptr_t)at_elem = rec;
             };
-            put(slot0, next.h0, hash, next.info0, next.rest0);
-            put(slot1, next.h1, hash, next.info1, next.rest1);
-            put(slots, hash, want, next.infos, next.rests);
+            put(slot0, next.h0, next.info0, next.rest0);
+            put(slot1, next.h1, next.info1, next.rest1);
+            put(slots, hash, next.infos, next.rests);
             wave_fence();
         }
         w = kept;
@@ -856,17 +851,18 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // their score and persist as zero, which is what the CPU path's untouched slots hold (a beam
         // cut below 1 empties the beam, and the traceback then walks such slots)
         {
-            const Elem e = sh.elem[i];
-            hash = e.hash;
-            want = e.want;
-            info = (uint32_t)pick_by_bit(vm, (int)e.info, 0);
-            score = __int_as_float(pick_by_bit(vm, __float_as_int(e.rest), __float_as_int(-FLT_MAX)));
+            typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+            const u32x3 e = *(const LDS_AS u32x3 *)(uintptr_t)((uint32_t)(uintptr_t)(lds_u32 *)&sh.elem[0].hash + 16u * (uint32_t)i);
+            hash = e.x;
+            info = (uint32_t)pick_by_bit(vm, (int)e.z, 0);
+            score = __int_as_float(pick_by_bit(vm, __float_as_int(__uint_as_float(e.y)), __float_as_int(-FLT_MAX)));
         }
         state = (int)(info & 1023u);
-        if (t + 1 < T) fetch_row(t + 1);
+        want = crc2_inverse(hash, (uint32_t)state & 3u);
+        if constexpr (!LAST) fetch_row(t + 1);
 
         // last block: the best survivor goes to slot 0 (src/beam_search.c:398-414)
-        if (t == T - 1) {
+        if constexpr (LAST) {
             const bool in = i < w;
             const float top_score = wave_max(score);
             const uint64_t at = ballot(in && h == 0 && score == top_score);
@@ -883,42 +879,118 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
         // that held the candidate, which had the term at hand.  Both halves hold the same element
         // and store the same slot; slots past the width are never followed by the traceback
         bv[(size_t)(t + 1) * kW + i] = (ofk_beam_slot_t)info;
-    }
+    };
+    for (int t = 0; t < T - 1; ++t) step(t, std::false_type{});
+    step(T - 1, std::true_type{});
 
     // ---- traceback from slot 0 of the last block (src/beam_search.c:432-439) ----
-    // The chase itself is serial: one LDS read per time step, its address taken from the slot
-    // read before.  Everything else is kept off that chain: the slot of row k of a round of 64
-    // rows is parked in lane k (a compare and a select over the whole wave; instructions that
-    // run with one lane enabled were measured to take three to five times as long as with all
-    // 64), and after the round every lane unpacks its own row and the wave stores 64 states and
-    // moves side by side.
+    // Followed one row at a time the walk is a chain of T dependent LDS reads.  It is done per block
+    // of 128 rows instead, staged in LDS (in the memory of the hash index, which is dead now), in two
+    // passes.  Pass 1 walks the block's eight sub-blocks of 16 rows at the same time, each from all
+    // 32 slots it could be entered through (lanes 0..31 the four newer sub-blocks, lanes 32..63 the
+    // four older ones): where every entry leaves its sub-block.  Eight lane reads then thread the
+    // real entry through the block.  Pass 2 walks the eight sub-blocks again, each from its real
+    // entry (eight lanes per sub-block, lane q keeping rows 2q and 2q+1 of the walk), and the
+    // wave stores 128 states and moves side by side.  Rows that a block lacks at its old end are
+    // staged as slots that point at themselves.  The next block's slots travel from global memory
+    // while a block is walked.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    int32_t *st_out = states + (size_t)n * T;
-    uint8_t *mv_out = moves + (size_t)n * T;
-    uint32_t cursor = 0;  // the same in every lane
-    for (int hi_t = T; hi_t > 0; hi_t -= TB) {
-        const int lo_t = hi_t > TB ? hi_t - TB : 0;  // rows lo_t+1 .. hi_t
-        const int rows = hi_t - lo_t;
-        const uint4 *src = reinterpret_cast<const uint4 *>(bv + (size_t)(lo_t + 1) * kW);
-        uint4 *dst = reinterpret_cast<uint4 *>(&trace[0][0]);
-        for (int x = lane; x < rows * 4; x += 64) dst[x] = src[x];  // 64 bytes per row
-        wave_fence();
-        for (int top = rows; top > 0; top -= 64) {
-            const int first = __builtin_amdgcn_readfirstlane(top > 64 ? top - 64 : 0);  // this round: rows first .. top-1, newest first
-            uint32_t mine = 0;
-            for (int r = top - 1; r >= first; --r) {
-                const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)trace[r][cursor]);
-                mine = lane == r - first ? e : mine;
-                cursor = (e >> 10) & 31u;
+    {
+        constexpr int RB = 128;  // rows per block
+        static_assert(2 * RB * kW * (int)sizeof(ofk_beam_slot_t) <= BeamIdx<S, CPG>::kBuckets * 8, "two blocks fit the index");
+        int32_t *st_out = states + (size_t)n * T;
+        uint8_t *mv_out = moves + (size_t)n * T;
+        const uint32_t buf0 = idx_base;  // two buffers of RB rows of 64 bytes, row 127 the newest of a block
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        u32x4 pre[8];  // a block on its way from global memory: 16-byte piece 64 k + lane in pre[k]
+        // block b covers rows hi - rows + 1 .. hi with hi = T - RB b; piece x of the buffer holds
+        // row x / 4 - (RB - rows) of those, or slots pointing at themselves before that
+        auto load_block = [&](int hi) {
+            const int rows = hi < RB ? hi : RB;
+            const u32x4 *src = reinterpret_cast<const u32x4 *>(bv + (size_t)(hi - rows + 1) * kW);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int x = 64 * k + lane - 4 * (RB - rows);
+                if (x >= 0) pre[k] = __builtin_nontemporal_load(src + x);
             }
-            const int t = lo_t + first + lane;
-            if (first + lane < top) {
-                st_out[t] = (int32_t)(mine & 1023u);
-                mv_out[t] = (t == 0 || !(mine >> 15)) ? (uint8_t)1 : (uint8_t)0;
+        };
+        auto store_block = [&](int hi, uint32_t buf) {
+            const int rows = hi < RB ? hi : RB;
+            const uint32_t c8 = (uint32_t)(lane & 3) * 8u;  // first of the eight slots of an identity piece
+            u32x4 self;
+            self.x = ((c8 + 0u) << 10) | ((c8 + 1u) << 26);
+            self.y = ((c8 + 2u) << 10) | ((c8 + 3u) << 26);
+            self.z = ((c8 + 4u) << 10) | ((c8 + 5u) << 26);
+            self.w = ((c8 + 6u) << 10) | ((c8 + 7u) << 26);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int x = 64 * k + lane - 4 * (RB - rows);
+                *(LDS_AS u32x4 *)(uintptr_t)(buf + 16u * (uint32_t)(64 * k + lane)) = x >= 0 ? pre[k] : self;
             }
+        };
+        auto slot_at = [&](uint32_t row_base, uint32_t cur, int row) {  // slot `cur` of row `row` above row_base
+            uint32_t at;
+            asm("v_lshl_add_u32 %0, %1, 1, %2" : "=v"(at) : "v"(cur), "v"(row_base));
+            return (uint32_t) * (const LDS_AS uint16_t *)(uintptr_t)(at + 64u * (uint32_t)row);
+        };
+        uint32_t cursor = 0;  // slot through which the walk enters the block: the same in every lane
+        load_block(T);
+        store_block(T, buf0);
+        int blk = 0;
+        for (int hi = T; hi > 0; hi -= RB, ++blk) {
+            const int rows = hi < RB ? hi : RB;
+            const uint32_t buf = buf0 + (uint32_t)(blk & 1) * (uint32_t)(RB * 64);
+            if (hi > RB) load_block(hi - RB);
+            wave_fence();
+            // pass 1: sub-block s = 4 (lane / 32) + k covers buffer rows 127 - 16 s down to 112 - 16 s
+            uint32_t cur[4];
+            const uint32_t low1 = buf + 64u * (uint32_t)(112 - 64 * (lane >> 5));  // oldest row of this lane's sub-block k = 0
+#pragma unroll
+            for (int k = 0; k < 4; ++k) cur[k] = (uint32_t)lane & 31u;
+#pragma unroll
+            for (int r = 15; r >= 0; --r) {
+                uint32_t e[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) e[k] = slot_at(low1 - (uint32_t)(16 * 64 * k), cur[k], r);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) cur[k] = (e[k] >> 10) & 31u;
+            }
+            // the real entry of every sub-block
+            uint32_t enter[8];
+#pragma unroll
+            for (int sb = 0; sb < 8; ++sb) {
+                enter[sb] = cursor;
+                cursor = (uint32_t)__builtin_amdgcn_readlane((int)cur[sb & 3], (int)(cursor + 32u * (uint32_t)(sb >> 2)));
+            }
+            // pass 2: lanes 8 s .. 8 s + 7 walk sub-block s from its real entry; lane q keeps rows 2q, 2q+1 of the walk
+            const int sb2 = lane >> 3, q = lane & 7;
+            uint32_t walk = enter[0];
+#pragma unroll
+            for (int sb = 1; sb < 8; ++sb) walk = sb2 == sb ? enter[sb] : walk;
+            const uint32_t low2 = buf + 64u * (uint32_t)(112 - 16 * sb2);
+            uint32_t newer = 0, older = 0;
+#pragma unroll
+            for (int r = 15; r >= 0; --r) {
+                const uint32_t e = slot_at(low2, walk, r);
+                if (r & 1) newer = q == (15 - r) / 2 ? e : newer;
+                else older = q == (15 - r) / 2 ? e : older;
+                walk = (e >> 10) & 31u;
+            }
+            // buffer row of `newer`: 127 - 16 sb2 - 2 q; the block's rows start at buffer row RB - rows,
+            // which is row hi - rows + 1 of the chunk, i.e. time step hi - rows
+            const int p_new = 127 - 16 * sb2 - 2 * q;
+            const int t_new = hi - rows + (p_new - (RB - rows));
+            if (p_new >= RB - rows) {
+                st_out[t_new] = (int32_t)(newer & 1023u);
+                mv_out[t_new] = (t_new == 0 || !(newer >> 15)) ? (uint8_t)1 : (uint8_t)0;
+            }
+            if (p_new - 1 >= RB - rows) {
+                st_out[t_new - 1] = (int32_t)(older & 1023u);
+                mv_out[t_new - 1] = (t_new - 1 == 0 || !(older >> 15)) ? (uint8_t)1 : (uint8_t)0;
+            }
+            if (hi > RB) store_block(hi - RB, buf0 + (uint32_t)((blk + 1) & 1) * (uint32_t)(RB * 64));
         }
-        wave_fence();
     }
 }
 
