@@ -912,7 +912,7 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
 #pragma unroll
             for (int k = 0; k < 8; ++k) {
                 const int x = 64 * k + lane - 4 * (RB - rows);
-                if (x >= 0) pre[k] = __builtin_nontemporal_load(src + x);
+                pre[k] = src[x > 0 ? x : 0];  // every lane loads (pieces before the block's first are not used)
             }
         };
         auto store_block = [&](int hi, uint32_t buf) {
@@ -977,6 +977,9 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 else older = q == (15 - r) / 2 ? e : older;
                 walk = (e >> 10) & 31u;
             }
+            // the next block goes into the other buffer before this block's results are stored: the wait
+            // for its loads then does not wait for those stores as well
+            if (hi > RB) store_block(hi - RB, buf0 + (uint32_t)((blk + 1) & 1) * (uint32_t)(RB * 64));
             // buffer row of `newer`: 127 - 16 sb2 - 2 q; the block's rows start at buffer row RB - rows,
             // which is row hi - rows + 1 of the chunk, i.e. time step hi - rows
             const int p_new = 127 - 16 * sb2 - 2 * q;
@@ -989,7 +992,6 @@ __global__ __launch_bounds__(128 * CPG) void beam_kernel(const _Float16 *__restr
                 st_out[t_new - 1] = (int32_t)(older & 1023u);
                 mv_out[t_new - 1] = (t_new - 1 == 0 || !(older >> 15)) ? (uint8_t)1 : (uint8_t)0;
             }
-            if (hi > RB) store_block(hi - RB, buf0 + (uint32_t)((blk + 1) & 1) * (uint32_t)(RB * 64));
         }
     }
 }
