@@ -23,7 +23,7 @@ HIPFLAGS := $(ROCM_ARCH) -O3 -fPIC -ffp-contract=off -Xclang -target-feature -Xc
 CFLAGS   := -O2 -g -Wall -fPIC -std=gnu11 -D__HIP_PLATFORM_AMD__ -I include -I $(SRC) -I $(ROCM_ROOT)/include
 LDLIBS   := -L$(ROCM_ROOT)/lib -Wl,-rpath,$(ROCM_ROOT)/lib -lamdhip64 -lm -lpthread
 
-HIP_OBJ := $(BUILD)/scan.o $(BUILD)/scan_five.o $(BUILD)/beam.o $(BUILD)/sequence.o $(BUILD)/rotary.o $(BUILD)/copy.o
+HIP_OBJ := $(BUILD)/scan.o $(BUILD)/scan_five.o $(BUILD)/beam.o $(BUILD)/sequence.o $(BUILD)/rotary.o $(BUILD)/copy.o $(BUILD)/probe.o
 C_OBJ   := $(BUILD)/openfish_host.o
 
 all: lib/libopenfish.a openfish_amd/libopenfish_amd.so openfish

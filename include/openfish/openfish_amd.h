@@ -101,19 +101,30 @@ void openfish_amd_beam_search(int T, int N, int C, const void *scores, int state
                               const openfish_gpubuf_t *gpubuf);
 
 /*
- * The same beam search and traceback for callers that must not allocate device memory (code
- * under HIP graph capture, tight serving loops): it has no counterpart in the reference.
- * Instead of a gpubuf it uses a static array of the library in device memory (64 MiB of beam
- * slots plus the log-sum-exp table, held by every GPU the library runs on until the process
- * ends) and writes its results to caller-provided device buffers: states int32 [N][T] (the
- * k-mer state of the traced path) and moves uint8 [N][T].  N * (T + 1) * 64 bytes must fit the
- * 64 MiB (hac at T = 1666: N <= 628), otherwise the call prints an error and exits.  It calls no
- * hipMalloc/hipFree; the first call on a device looks up the array's address and copies the
- * 4.9 KB table into it.  All calls on one GPU share the array: calls that overlap in time race.
+ * The same beam search and traceback for callers that must not allocate device memory while they
+ * run (tight serving loops, harnesses that forbid it, code that records its launches on a stream):
+ * it has no counterpart in the reference.  Instead of a gpubuf it uses a static array of the
+ * library in device memory (64 MiB of beam slots plus the log-sum-exp table, held by every GPU the
+ * library runs on until the process ends) and writes its results to caller-provided device
+ * buffers: states int32 [N][T] (the k-mer state of the traced path) and moves uint8 [N][T].
+ *
+ * openfish_amd_beam_search_static_prepare() sets the array up on the current device, once: it looks
+ * up the array's address and copies the 4.9 KB table into it with a blocking copy (not for use
+ * inside a stream capture; later calls on the same device return at once).
+ *
+ * openfish_amd_beam_search_static(...) then only launches the kernel on `stream` (NULL: the null
+ * stream) and returns without waiting: it calls no hipMalloc/hipFree, no copy and no
+ * synchronisation; the results are valid once the stream has reached the launch.  It exits with a
+ * message if the device has not been prepared, or if N * (T + 1) * 64 bytes exceed the 64 MiB (hac
+ * at T = 1666: N <= 628).  All calls on one GPU share the array: calls that overlap in time race.
  */
+void openfish_amd_beam_search_static_prepare(void);
 void openfish_amd_beam_search_static(int T, int N, int C, const void *scores, int state_len,
                                      const openfish_opt_t *options, const float *bwd, int32_t *states,
-                                     uint8_t *moves);
+                                     uint8_t *moves, void *stream);
+
+/* free device memory in bytes (hipMemGetInfo): lets a test see that a call allocated nothing */
+size_t openfish_amd_device_free_bytes(void);
 
 /*
  * Per-block quality, base calls and phred string (reference src/beam_search.c:441-496
@@ -219,6 +230,19 @@ void openfish_amd_phred_table(float q_scale, float q_shift, float *thr49);
  * s = 8 * (gap - cell centre).  Writes 612 doubles.  Host-only; needs no device.
  */
 void openfish_amd_lse_table(double *out);
+
+/*
+ * Measures, on the current device, the worst error of the two hardware transcendentals the
+ * default scan arithmetic and the beam search's merges build on, over every fp32 input of the
+ * ranges they are used on, against double arithmetic; in units of 2^-24:
+ *   errors4[0]  v_exp_f32, largest relative error over [-160, 0] (results in the normal range)
+ *   errors4[1..3]  v_log_f32, largest absolute error over [1, 2), [2, 4), [4, 5.01]
+ * identities: bit 0 exp2(0) == 1, bit 1 exp2(-0) == 1, bit 2 log2(1) == 0, bit 3 log2(2) == 1.
+ * The two-tier evaluations are exact while these stay within 1.43, 1.0, 2.0, 4.0 and all four
+ * identities hold (csrc/dmath.h, csrc/beam.hip); a test asserts that on the device at hand.
+ * No counterpart in the reference, whose GPU path makes no claim of bit-exactness.
+ */
+void openfish_amd_probe_hw_math(double *errors4, unsigned int *identities);
 
 /* library build tag, e.g. "openfish-amd gfx950" */
 const char *openfish_amd_version(void);

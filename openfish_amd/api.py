@@ -81,7 +81,9 @@ _SIGS = {
     "openfish_amd_scan_posterior": (None, [_i, _i, _i, _vp, _i, _f, _i, _vp, _vp]),
     "openfish_amd_gpubuf_set_split_scans": (None, [_bufp, _i]),
     "openfish_amd_beam_search": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _bufp]),
-    "openfish_amd_beam_search_static": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _vp, _vp]),
+    "openfish_amd_beam_search_static_prepare": (None, []),
+    "openfish_amd_beam_search_static": (None, [_i, _i, _i, _vp, _i, _optp, _vp, _vp, _vp, _vp]),
+    "openfish_amd_device_free_bytes": (_sz, []),
     "openfish_amd_sequence": (None, [_i, _i, _i, _optp, _vp, _bufp]),
     "openfish_amd_decode_enqueue": (None, [_i, _i, _i, _vp, _i, _optp, _bufp]),
     "openfish_amd_decode_wait": (None, [_bufp, _pp, _pp, _pp]),
@@ -92,6 +94,7 @@ _SIGS = {
     "openfish_amd_gpubuf_set_scan_states_per_lane": (None, [_bufp, _i]),
     "openfish_amd_lse_table": (None, [C.POINTER(C.c_double)]),
     "openfish_amd_phred_table": (None, [_f, _f, C.POINTER(C.c_float)]),
+    "openfish_amd_probe_hw_math": (None, [C.POINTER(C.c_double), C.POINTER(C.c_uint)]),
     "openfish_amd_version": (C.c_char_p, []),
 }
 
@@ -285,10 +288,21 @@ def openfish_amd_beam_search(T, N, Cc, scores_dev, state_len, options, bwd_dev, 
     _L.openfish_amd_beam_search(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), _ptr(bwd_dev), gpubuf.handle)
 
 
-def openfish_amd_beam_search_static(T, N, Cc, scores_dev, state_len, options, bwd_dev, states_dev, moves_dev):
-    """the beam search on the library's static scratch array: allocates nothing"""
+def openfish_amd_beam_search_static_prepare():
+    """set up the library's static scratch array on the current device (once; blocking)"""
+    _L.openfish_amd_beam_search_static_prepare()
+
+
+def openfish_amd_beam_search_static(T, N, Cc, scores_dev, state_len, options, bwd_dev, states_dev, moves_dev,
+                                    stream=None):
+    """the beam search on the library's static scratch array: launches on `stream` and returns;
+    allocates nothing, copies nothing, waits for nothing (openfish_amd_sync() before reading results)"""
     _L.openfish_amd_beam_search_static(T, N, Cc, _ptr(scores_dev), state_len, C.byref(options), _ptr(bwd_dev),
-                                       _ptr(states_dev), _ptr(moves_dev))
+                                       _ptr(states_dev), _ptr(moves_dev), stream)
+
+
+def device_free_bytes():
+    return int(_L.openfish_amd_device_free_bytes())
 
 
 def openfish_amd_sequence(T, N, state_len, options, post_dev, gpubuf):
@@ -311,6 +325,14 @@ def phred_table(q_scale, q_shift):
     thr = (C.c_float * 49)()
     _L.openfish_amd_phred_table(q_scale, q_shift, thr)
     return np.array(thr[:], dtype=np.float32)
+
+
+def probe_hw_math():
+    """(errors in units of 2^-24: exp on [-160,0], log on [1,2), [2,4), [4,5.01]; identity bits)"""
+    err = (C.c_double * 4)()
+    ident = C.c_uint(0)
+    _L.openfish_amd_probe_hw_math(err, C.byref(ident))
+    return [float(x) for x in err], int(ident.value)
 
 
 def lse_table():

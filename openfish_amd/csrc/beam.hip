@@ -261,7 +261,8 @@ __device__ __forceinline__ float log_sum_exp(float x, float y, const double *tab
 //   1.00  1 + e rounded to fp32
 //   1.39  v_log_f32 on [1, 2] (largest absolute error over every input: 1.0 below 2, 2.0 at 2), times ln 2
 //   0.08  ln2f against ln 2, the rounding of the residual
-// together 3.64; the bound used is 4.0.  The result is settled when the distance from the
+// together 3.64; the bound used is 4.0.  (The two hardware figures are measured on the device at
+// hand, over every fp32 input of their ranges, by tests/test_gpu_hw_math.py.)  The result is settled when the distance from the
 // unrounded sum to the nearer rounding boundary of the result exceeds that bound (the residual of
 // the fused multiply-add, taken exactly with a second one).  Half an ulp is read from the exponent
 // of the next smaller float, which for a power of two is the binade below, where its nearer
@@ -1050,10 +1051,37 @@ std::mutex g_scratch_mutex;
 
 }  // namespace
 
+// Set-up of the static scratch array on the current device: looks up the array's device address and
+// copies the log-sum-exp table behind it (a blocking copy).  Once per device; later calls return at once.
+extern "C" int ofk_beam_search_static_prepare(const double *lse_table_host) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return OFK_BAD_ARGS;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_of[dev]) return 0;
+    if (!lse_table_host) return OFK_BAD_ARGS;
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    e = hipMemcpy(p, lse_table_host, sizeof(double) * OFK_LSE_DOUBLES, hipMemcpyHostToDevice);
+    if (e != hipSuccess) return (int)e;
+    g_scratch_of[dev] = static_cast<unsigned char *>(p);
+    return 0;
+}
+
+// 1 if the current device's array has been set up, 0 if not (or if the device cannot be told)
+extern "C" int ofk_beam_search_static_ready(void) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    return g_scratch_of[dev] ? 1 : 0;
+}
+
 extern "C" int ofk_beam_search_static(const void *scores, const float *bwd, int32_t *states, uint8_t *moves, int T,
-                                      int N, int state_len, int columns, float log_beam_cut, float stay,
-                                      const double *lse_table_host, int flags, void *stream) {
-    if (!scores || !bwd || !states || !moves || !lse_table_host || T < 1 || N < 1) return OFK_BAD_ARGS;
+                                      int N, int state_len, int columns, float log_beam_cut, float stay, int flags,
+                                      void *stream) {
+    if (!scores || !bwd || !states || !moves || T < 1 || N < 1) return OFK_BAD_ARGS;
     if ((reinterpret_cast<uintptr_t>(scores) | reinterpret_cast<uintptr_t>(bwd)) & 15u) return OFK_BAD_ARGS;
     if ((size_t)N * (size_t)(T + 1) * kW * sizeof(ofk_beam_slot_t) > (size_t)OFK_STATIC_SLOT_BYTES) return OFK_TOO_LARGE;
     int dev = -1;
@@ -1062,18 +1090,10 @@ extern "C" int ofk_beam_search_static(const void *scores, const float *bwd, int3
     if (dev < 0 || dev >= kMaxDevices) return OFK_BAD_ARGS;
     unsigned char *base;
     {
-        // set-up, once per device: the array's device address, and the table copied behind it
         std::lock_guard<std::mutex> lock(g_scratch_mutex);
-        if (!g_scratch_of[dev]) {
-            void *p = nullptr;
-            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-            if (e != hipSuccess) return (int)e;
-            e = hipMemcpy(p, lse_table_host, sizeof(double) * OFK_LSE_DOUBLES, hipMemcpyHostToDevice);
-            if (e != hipSuccess) return (int)e;
-            g_scratch_of[dev] = static_cast<unsigned char *>(p);
-        }
         base = g_scratch_of[dev];
     }
+    if (!base) return OFK_NOT_PREPARED;
     // nothing in the array has to start at zero: the search writes every slot the traceback reads
     ofk_beam_slot_t *beam = reinterpret_cast<ofk_beam_slot_t *>(base + kStaticTableBytes);
     const double *lse_table = reinterpret_cast<const double *>(base);

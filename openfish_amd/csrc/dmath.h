@@ -229,7 +229,10 @@ OFA_HD float lse5_cpu_rounding_tab(float v0, float v1, float v2, float v3, float
 // function), so that
 //   eps = 14.13 - 8.5 mu + 1.045 * 2^k    (11.0 at s~ = 1, 6.7 just below 2, 12.0 at 2, ...)
 // is a bound, evaluated from the bits of s~ with two fused multiply-adds; the constants below
-// add 3 %.  The binade is read from s~ raised by 16 ulps: should s_cpu, within a dozen ulps
+// add 3 %.  The four hardware figures (1.43 for v_exp_f32; 1.0, 2.0, 4.0 for v_log_f32) and the
+// identities exp2(0) = 1, log2(1) = 0 are premises about the device: tests/test_gpu_hw_math.py
+// measures them over every fp32 input of those ranges on the device it runs on (probe.hip) and
+// fails if one is exceeded.  The binade is read from s~ raised by 16 ulps: should s_cpu, within a dozen ulps
 // of s~, reach the next binade, where half an ulp is twice as large, s~ counts as being there too.
 //
 // r~ is settled when no rounding boundary lies within eps of x~: with rho = x~ - r~ (exact up

@@ -57,13 +57,17 @@ int ofk_beam_search(const void *scores, const float *bwd, ofk_beam_slot_t *beam,
                     const double *lse_table, int flags, void *stream);
 /* The same search with the beam slots and the table in a static device array of the library
  * (OFK_STATIC_SLOT_BYTES of slots: N * (T + 1) * 64 bytes must fit, else OFK_TOO_LARGE and nothing
- * is launched).  Allocates nothing; the first call on a device looks up the array's address and
- * copies the 612 doubles at lse_table_host (host memory) into it.  Calls that overlap in time on
- * one device share the array and race. */
+ * is launched).  ofk_beam_search_static_prepare sets the array up on the current device (looks up
+ * its address, copies the 612 doubles at lse_table_host, host memory, into it with a blocking
+ * copy; a no-op once done).  ofk_beam_search_static then only launches the kernel on `stream`: it
+ * allocates nothing, copies nothing and waits for nothing (OFK_NOT_PREPARED if the device's array
+ * has not been set up).  Calls that overlap in time on one device share the array and race. */
 #define OFK_STATIC_SLOT_BYTES (64u << 20)
+#define OFK_NOT_PREPARED (-3)
+int ofk_beam_search_static_prepare(const double *lse_table_host);
+int ofk_beam_search_static_ready(void);
 int ofk_beam_search_static(const void *scores, const float *bwd, int32_t *states, uint8_t *moves, int T, int N,
-                           int state_len, int columns, float log_beam_cut, float stay, const double *lse_table_host,
-                           int flags, void *stream);
+                           int state_len, int columns, float log_beam_cut, float stay, int flags, void *stream);
 /* flags, for tests.  Bit 0: replay every stay/step merge one by one in CPU order (the path
  * otherwise taken only after a hash collision); results must not change.  Bit 1: seed hashes are
  * taken from (state & 15), so that different sequences share hashes and the search has to notice
@@ -84,6 +88,13 @@ int ofk_copy(void *dst, const void *src, size_t bytes, void *stream);
 int ofk_rotary_emb(void *x, const float *sin_buf, const float *cos_buf, int batch, int seqlen,
                    int nheads, int rotary_half, long stride_batch, long stride_seq, long stride_head,
                    void *stream);
+
+/* Worst errors of v_exp_f32 over every fp32 in [-160, 0] (relative, results in the normal range)
+ * and of v_log_f32 over every fp32 in [1, 2), [2, 4), [4, 5.01] (absolute), against double
+ * arithmetic, plus the identities exp2(0) = exp2(-0) = 1, log2(1) = 0, log2(2) = 1.  The results
+ * go to 40 bytes of device memory at scratch40 (8-byte aligned): four doubles, then a word of
+ * identity bits (bit 0..3 in the order above). */
+int ofk_probe_hw_math(void *scratch40, void *stream);
 
 #ifdef __cplusplus
 }

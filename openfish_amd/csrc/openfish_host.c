@@ -2,10 +2,10 @@
  * Host side of the MI355X decoder: the public openfish entry points and the
  * stage-level C-ABI, in C, above the kernel launchers of kernels.h.
  *
- * One decode is   bwd scan -> { beam search || fwd+posterior scan } -> sequence.
- * The beam search needs only scores and bwd, the posterior only feeds the quality
- * stage (reference src/beam_search.c:193,450), so the two run on two streams and
- * share the device.  Errors follow the reference convention (reference
+ * One decode is   scans + posterior (one kernel) -> beam search -> sequence   on one stream, or,
+ * for very large batches and on request,   bwd scan -> { beam search || fwd+posterior scan } ->
+ * sequence   on two (the beam search needs only scores and bwd, the posterior only feeds the
+ * quality stage, reference src/beam_search.c:193,450).  Errors follow the reference convention (reference
  * src/hip_utils.h:11-28, src/error.h:44-72): message on stderr, then exit.
  */
 #include <errno.h>
@@ -519,16 +519,22 @@ void openfish_amd_beam_search(int T, int N, int C, const void *scores, int state
     HIP_OK(hipStreamSynchronize(0));
 }
 
+void openfish_amd_beam_search_static_prepare(void) {
+    if (ofk_beam_search_static_ready()) return;
+    double tab[OFK_LSE_DOUBLES];
+    build_lse_table(tab);
+    launch_ok(ofk_beam_search_static_prepare(tab), "beam_search_static_prepare");
+}
+
 void openfish_amd_beam_search_static(int T, int N, int C, const void *scores, int state_len,
                                      const openfish_opt_t *options, const float *bwd, int32_t *states,
-                                     uint8_t *moves) {
+                                     uint8_t *moves, void *stream) {
     check_scores(T, N, C, scores, state_len, options);
     if (!bwd || !states || !moves) die("beam_search_static: bwd, states and moves must be device pointers");
-    double tab[OFK_LSE_DOUBLES]; /* read by the first call on a device only */
-    build_lse_table(tab);
     const int rc = ofk_beam_search_static(scores, bwd, states, moves, T, N, state_len, columns_of(C, state_len),
-                                          log_beam_cut(options),
-                                          options->blank_score, tab, 0, NULL);
+                                          log_beam_cut(options), options->blank_score, 0, stream);
+    if (rc == OFK_NOT_PREPARED)
+        die("beam_search_static: call openfish_amd_beam_search_static_prepare() on this device first");
     if (rc == OFK_TOO_LARGE) {
         fprintf(stderr, "openfish: beam_search_static: N * (T + 1) * 64 = %zu bytes of beam slots exceed the static "
                         "scratch array of %u bytes; use openfish_amd_beam_search with a gpubuf\n",
@@ -536,7 +542,12 @@ void openfish_amd_beam_search_static(int T, int N, int C, const void *scores, in
         exit(EXIT_FAILURE);
     }
     launch_ok(rc, "beam_search_static");
-    HIP_OK(hipStreamSynchronize(0));
+}
+
+size_t openfish_amd_device_free_bytes(void) {
+    size_t free_b = 0, total_b = 0;
+    HIP_OK(hipMemGetInfo(&free_b, &total_b));
+    return free_b;
 }
 
 void openfish_amd_sequence(int T, int N, int state_len, const openfish_opt_t *options, const float *post,
@@ -644,6 +655,20 @@ void openfish_amd_sync(void) { HIP_OK(hipDeviceSynchronize()); }
 void openfish_amd_copy(void *dst, const void *src, size_t bytes) {
     launch_ok(ofk_copy(dst, src, bytes, NULL), "copy");
     HIP_OK(hipStreamSynchronize(0));
+}
+
+void openfish_amd_probe_hw_math(double *errors4, unsigned int *identities) {
+    if (!errors4 || !identities) die("probe_hw_math: output pointer is NULL");
+    void *dev = NULL;
+    unsigned char host[40];
+    HIP_OK(hipMalloc(&dev, sizeof host));
+    launch_ok(ofk_probe_hw_math(dev, NULL), "probe_hw_math");
+    HIP_OK(hipStreamSynchronize(0));
+    HIP_OK(hipMemcpy(host, dev, sizeof host, hipMemcpyDeviceToHost));
+    HIP_OK(hipFree(dev));
+    memcpy(errors4, host, 4 * sizeof(double));
+    memcpy(identities, host + 32, sizeof *identities);
+    for (int k = 0; k < 4; ++k) errors4[k] *= 16777216.0; /* in units of 2^-24 */
 }
 
 int openfish_amd_device_count(void) {

@@ -145,23 +145,9 @@ struct LogArgs {
 // result returns to its owner through a lane permute.  More than eight unsettled lanes take
 // further trips (only the first few dozen time steps have that many: values are small there and
 // an ulp is tiny; the kernels run those steps with the double arithmetic throughout).
-#ifdef OFK_TIER_STATS
-// build with -DOFK_TIER_STATS to count, per wave-level update of the two-tier scans: updates, updates
-// with unsettled lanes, second-tier trips, unsettled lanes (read with ofk_tier_stats)
-__device__ unsigned long long g_tier_stats[4];
-#endif
-
 __device__ __forceinline__ float resolve_unsettled(float value, float sum, bool unsettled, float v0, float v1, float v2,
                                                    float v3, float v4, float m, const LogArgs &logtab) {
     uint64_t mask = __builtin_amdgcn_ballot_w64(unsettled);
-#ifdef OFK_TIER_STATS
-    if ((threadIdx.x & 63) == 0) {
-        atomicAdd(&g_tier_stats[0], 1ull);
-        if (mask) atomicAdd(&g_tier_stats[1], 1ull);
-        atomicAdd(&g_tier_stats[2], (unsigned long long)((__builtin_popcountll(mask) + 7) / 8));
-        atomicAdd(&g_tier_stats[3], (unsigned long long)__builtin_popcountll(mask));
-    }
-#endif
     if (mask == 0) return value;
     __builtin_amdgcn_s_setprio(3);  // the chunk's other waves wait at the barrier for this one
     const int lane = threadIdx.x & 63;
@@ -1047,9 +1033,6 @@ int states_per_lane(int S, int N, bool backward, int forced) {
 // 64 states need one state per lane; as many lanes as it takes to put four waves on every SIMD,
 // within the 1024 threads of a workgroup.
 static int fused_states_per_lane(int S, int N, int forced) {
-#ifdef OFK_FORCE_FUSED_SPL
-    if (S == 256) forced = OFK_FORCE_FUSED_SPL;
-#endif
     const int min_spl = S >= 1024 ? 2 : 1, max_spl = S >= 256 ? 4 : 1;
     if (forced == 4 || forced == 2 || forced == 1) return forced < min_spl ? min_spl : (forced > max_spl ? max_spl : forced);
     for (int spl = max_spl; spl > min_spl; spl >>= 1) {
@@ -1058,17 +1041,6 @@ static int fused_states_per_lane(int S, int N, int forced) {
     }
     return min_spl;
 }
-
-#if defined(OFK_TIER_STATS) && OFK_COLS == 4
-extern "C" void ofk_tier_stats(unsigned long long *out, int reset) {
-    (void)hipDeviceSynchronize();
-    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_tier_stats), sizeof(unsigned long long) * 4);
-    if (reset) {
-        unsigned long long z[4] = {0, 0, 0, 0};
-        (void)hipMemcpyToSymbol(HIP_SYMBOL(g_tier_stats), z, sizeof z);
-    }
-}
-#endif
 
 static int scan_posterior(const void *scores, float *bwd, float *post, int T, int N, int state_len, float stay,
                           int mode, int spl, void *stream) {

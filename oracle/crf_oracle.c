@@ -13,7 +13,13 @@
 #include <stdlib.h>
 #include <string.h>
 
-#define STAY_SCORE_SCAN 2.0f /* the CPU scans ignore opt->blank_score (src/decode_cpu.c:14,56) */
+/* The CPU scans ignore opt->blank_score and add the literal 2.0f for a stay (src/decode_cpu.c:14,56);
+ * the reference's GPU scans add opt->blank_score (src/decode_hip.hip:120).  The default below is the
+ * CPU path's; ofo_set_scan_stay is a test knob that puts another value in its place, so that the
+ * GPU scans can be compared at other blank scores. */
+static float g_scan_stay = 2.0f;
+#define STAY_SCORE_SCAN g_scan_stay
+void ofo_set_scan_stay(float stay) { g_scan_stay = stay; }
 #define CRC_POLY 0x82f63b78u /* reflected Castagnoli polynomial */
 #define CRC_SEED 0x12345678u /* src/decode.h:54 */
 

@@ -11,6 +11,11 @@
  *       pinned: bit-for-bit against the compiled reference (oracle/_ref) on
  *       seeded inputs; closed form for constant scores; brute-force path
  *       enumeration for state_len 1; row sums of the posterior.
+ *       With ofo_set_scan_stay at a value other than the reference CPU path's literal 2.0 (the
+ *       reference's GPU scans take options->blank_score there, src/decode_hip.hip:120) no
+ *       reference vector exists; that setting is pinned by the closed form
+ *       (T-t) log(e^stay + 4 e^c) on constant scores and by dense transition-matrix products
+ *       with e^stay on the diagonal (tests/test_oracle.py).
  *   ofo_crc32c            pinned: CRC-32C check value 0xE3069283 of "123456789".
  *   ofo_kth_largest       pinned: equals sort(desc)[k] on random and tied input.
  *   ofo_log_sum_exp       pinned: log(e^x+e^y) closed form, 17.0 cut-off.
@@ -69,6 +74,9 @@ typedef struct {
 uint32_t ofo_crc32c(uint32_t crc, uint32_t bits, int nbits);
 float ofo_kth_largest(float *v, int k, int n);
 float ofo_log_sum_exp(float x, float y);
+
+/* test knob: the stay score the scans add (default: the reference CPU path's literal 2.0f).  Process-wide. */
+void ofo_set_scan_stay(float stay);
 
 /* scans over one chunk; scores is the fp32 [T][N][4S] tensor */
 void ofo_backward_scan(const float *scores, float *bwd, size_t chunk, size_t T, size_t N, size_t S);

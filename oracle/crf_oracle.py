@@ -55,6 +55,8 @@ def lib():
         L.ofo_crc32c.argtypes = [C.c_uint32, C.c_uint32, C.c_int]
         L.ofo_set_seed_state_mask.restype = None
         L.ofo_set_seed_state_mask.argtypes = [C.c_uint32]
+        L.ofo_set_scan_stay.restype = None
+        L.ofo_set_scan_stay.argtypes = [C.c_float]
         L.ofo_kth_largest.restype = C.c_float
         L.ofo_kth_largest.argtypes = [f32p, C.c_int, C.c_int]
         L.ofo_log_sum_exp.restype = C.c_float
@@ -84,6 +86,13 @@ def set_seed_state_mask(mask=0xFFFFFFFF):
     """test knob: seed hashes from (state & mask); a narrow mask makes sequences share hashes.
     Reset it (no argument) when done: the setting is process-wide."""
     lib().ofo_set_seed_state_mask(mask & 0xFFFFFFFF)
+
+
+def set_scan_stay(stay=2.0):
+    """test knob: the stay score the scans add.  The reference CPU path adds the literal 2.0 whatever
+    options->blank_score says (src/decode_cpu.c:14,56); its GPU scans add blank_score
+    (src/decode_hip.hip:120).  Reset it (no argument) when done: the setting is process-wide."""
+    lib().ofo_set_scan_stay(C.c_float(stay))
 
 
 def kth_largest(values, k):

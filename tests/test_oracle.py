@@ -85,10 +85,10 @@ def test_scans_constant_scores_closed_form(state_len):
     np.testing.assert_allclose(post, 1.0 / S, rtol=1e-5)
 
 
-def transition_matrices(sc64, state_len):
+def transition_matrices(sc64, state_len, stay=2.0):
     """dense per-step matrices from the k-mer definition: from k-mer p a step
     appends base b giving s = ((p<<2) & mask) | b, scored by entry s*4 + (leading
-    base of p); staying in p scores 2.0"""
+    base of p); staying in p scores `stay` (2.0 on the reference CPU path)"""
     T, C = sc64.shape
     S = 4 ** state_len
     M = np.zeros((T, S, S))
@@ -97,7 +97,7 @@ def transition_matrices(sc64, state_len):
         for b in range(4):
             s = ((p << 2) & (S - 1)) | b
             M[:, p, s] += np.exp(sc64[:, s * 4 + lead])
-        M[:, p, p] += np.exp(2.0)
+        M[:, p, p] += np.exp(stay)
     return M
 
 
@@ -124,6 +124,47 @@ def test_scans_against_dense_matrix_products(state_len, T):
         np.testing.assert_allclose(fwd[n], want_f + want_b, rtol=1e-5, atol=1e-5)
         joint = np.exp(want_f + want_b - (want_f + want_b).max(axis=1, keepdims=True))
         np.testing.assert_allclose(post[n], joint / joint.sum(axis=1, keepdims=True), rtol=1e-4, atol=1e-7)
+
+
+@pytest.mark.parametrize("stay", [0.5, -1.5, 5.0])
+def test_scan_stay_knob_against_closed_form_and_dense_products(stay):
+    """the oracle's scans with another stay score than the CPU path's 2.0 (what the reference's GPU
+    scans do with options->blank_score, src/decode_hip.hip:120): closed form on constant scores,
+    and dense transition-matrix products with e^stay on the diagonal"""
+    O.set_scan_stay(stay)
+    try:
+        T, N, sl, c = 40, 2, 3, -0.25
+        S = 4 ** sl
+        bwd, fwd, post = O.scans(np.full((T, N, 4 * S), c, np.float32), sl)
+        per_step = np.log(np.exp(stay) + 4 * np.exp(c))
+        want = (T - np.arange(T + 1)) * per_step
+        np.testing.assert_allclose(bwd, np.broadcast_to(want[None, :, None], bwd.shape), rtol=2e-6, atol=1e-6)
+        np.testing.assert_allclose(fwd, T * per_step, rtol=2e-6)
+        np.testing.assert_allclose(post, 1.0 / S, rtol=1e-5)
+        T = 12
+        s32 = synth.crf_scores(T, N, sl, seed=5).astype(np.float32)
+        bwd, fwd, post = O.scans(s32, sl)
+        for n in range(N):
+            M = transition_matrices(s32[:, n, :].astype(np.float64), sl, stay)
+            beta = np.ones(S)
+            want_b = [np.zeros(S)]
+            for t in range(T - 1, -1, -1):
+                beta = M[t] @ beta
+                want_b.append(np.log(beta))
+            want_b = np.array(want_b[::-1])
+            np.testing.assert_allclose(bwd[n], want_b, rtol=1e-5, atol=1e-5)
+            alpha = np.ones(S)
+            want_f = [np.zeros(S)]
+            for t in range(T):
+                alpha = alpha @ M[t]
+                want_f.append(np.log(alpha))
+            want_f = np.array(want_f)
+            np.testing.assert_allclose(fwd[n], want_f + want_b, rtol=1e-5, atol=1e-5)
+    finally:
+        O.set_scan_stay()
+    # back at the CPU path's literal: the default scans are the golden-pinned ones again
+    bwd2, _, _ = O.scans(np.full((8, 1, 4 * 64), 0.5, np.float32), 3)
+    np.testing.assert_allclose(bwd2[0, 0, 0], 8 * np.log(np.exp(2.0) + 4 * np.exp(0.5)), rtol=2e-6)
 
 
 def test_state_len1_brute_force_paths():

@@ -1,6 +1,7 @@
 """The beam search entry point that allocates nothing (its scratch is a static device array of
 the library) against the entry point that works on a gpubuf, through the C-ABI: same states and
-moves, bit for bit, on two calls in a row, the second one smaller."""
+moves, bit for bit, on two calls in a row, the second one smaller; and the amount of free device
+memory is the same before and after a call."""
 import numpy as np
 import pytest
 
@@ -35,7 +36,12 @@ def both_entry_points(api, state_len, T, N, seed, scale=None, columns=4, **opt_k
     states, moves = api.DeviceBuffer(4 * N * T), api.DeviceBuffer(N * T)
     states.fill(0xEE)
     moves.fill(0xEE)
-    api.openfish_amd_beam_search_static(T, N, C, sc, state_len, opt, bwd, states, moves)
+    api.openfish_amd_beam_search_static_prepare()  # once per device; later calls return at once
+    api.lib().openfish_amd_sync()
+    free_before = api.device_free_bytes()
+    api.openfish_amd_beam_search_static(T, N, C, sc, state_len, opt, bwd, states, moves)  # launches and returns
+    api.lib().openfish_amd_sync()
+    assert api.device_free_bytes() == free_before, "the call changed the amount of free device memory"
     got_states, got_moves = states.to_host(np.int32, (N, T)), moves.to_host(np.uint8, (N, T))
     assert np.array_equal(got_moves, want_moves)
     assert np.array_equal(got_states, want_states)
