@@ -631,6 +631,13 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
     constexpr int RW = Sh::kRoleWaves;
     constexpr int H4 = 4 / SPL;  // backward lanes sharing one quad
     constexpr int kWarmup = 32;  // time steps of either sweep evaluated in double before the two tiers take over
+    // Per time step the lanes of one direction exchange their state vector (and the partial sums of
+    // the posterior's denominator) through LDS.  With several waves per direction that takes a
+    // workgroup barrier, which both directions (and every chunk of the group) then share; when a
+    // direction is a single wave (64 states), a time step only needs the wave's own LDS operations
+    // kept in order, and the waves of a group run their steps without waiting for one another.  The
+    // two directions of a chunk meet only in the middle, at block barriers that every wave reaches.
+    auto step_sync = [] { chunk_sync<(RW > 1)>(); };
     using VecB = BwdVec<S>;
     __shared__ __attribute__((aligned(16))) float vecB[Sh::kChunks][2][VecB::kLen];
     __shared__ __attribute__((aligned(16))) float vecF[Sh::kChunks][2][S];
@@ -696,7 +703,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                     ring[k].load(pre + sc_lane);
                     pre -= row_stride;
                 }
-                block_barrier_lds();
+                step_sync();
                 const float4 nx = *reinterpret_cast<const float4 *>(&vecB[g][buf][VecB::of(4 * r)]);
                 bwd_update<0, SPL, M>(a, nx, row, stay, logtab);
                 buf ^= 1;
@@ -750,7 +757,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                     pre -= row_stride;
                     fpre -= S;
                 }
-                block_barrier_lds();
+                step_sync();
                 if (j > 0) {  // posterior of the previous row: its total is complete now
                     float total = part[g][0][pb ^ 1][0];
 #pragma unroll
@@ -782,7 +789,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                 orow -= S;
             });
         }
-        block_barrier_lds();
+        step_sync();
         if (cnt2 > 0) {
             float total = part[g][0][pb ^ 1][0];
 #pragma unroll
@@ -794,7 +801,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
             }
         }
         // the forward lanes take T - H + 1 barriers in phase 2, these took H + 1
-        for (int x = H + 1; x < T - H + 1; ++x) block_barrier_lds();
+        for (int x = H + 1; x < T - H + 1; ++x) step_sync();
     } else {
         // ------------------------------ forward lanes ------------------------------
         const int s0 = SPL * l, q = s0 >> 2;  // own states s0 .. s0+SPL-1, all in quad q
@@ -835,7 +842,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                     mine.store(prow + st_lane);
                 }
                 prow += S;
-                block_barrier_lds();
+                step_sync();
                 const float p0 = vecF[g][buf][q], p1 = vecF[g][buf][q + Q];
                 const float p2 = vecF[g][buf][q + 2 * Q], p3 = vecF[g][buf][q + 3 * Q];
                 fwd_update<0, SPL, M>(f, p0, p1, p2, p3, row, stay, logtab);
@@ -849,7 +856,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
         const int warm = MODE == OFK_SCAN_TWO_TIER ? (cnt1 < kWarmup ? cnt1 : kWarmup) : 0;
         if constexpr (MODE == OFK_SCAN_TWO_TIER) sweep1(std::integral_constant<int, OFK_SCAN_PRECISE>{}, 0, warm);
         sweep1(std::integral_constant<int, MODE>{}, warm, cnt1 - warm);
-        for (int x = cnt1; x < T - H; ++x) block_barrier_lds();  // the backward lanes' extra step
+        for (int x = cnt1; x < T - H; ++x) step_sync();  // the backward lanes' extra step
 
         // middle: shift = max_s(fwd[H][s] + bwd[H][s]) - 10
         __syncthreads();
@@ -901,7 +908,7 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
                 }
                 total = group_sum<64>(total);
                 if ((tid & 63) == 0) part[g][1][pb][wave] = total;
-                block_barrier_lds();
+                step_sync();
                 total = part[g][1][pb][0];
 #pragma unroll
                 for (int w = 1; w < RW; ++w) total += part[g][1][pb][w];
