@@ -93,6 +93,34 @@ def cpu_baseline(s16, state_len, opt_kw, sample_chunks):
                       "median of 3 calls of openfish_decode_cpu (%.3f s each)" % (sample_chunks, T, sec)}
 
 
+def cpu_baseline_config1(seed):
+    """BASELINE's first configuration, the one the reference runs on the CPU: fast model (state_len 3,
+    64 states), T=1666, N=16 chunks, fp32 scores (the fp16-rounded values of the generator), beam 32,
+    beam cut 100, blank 2.0, q_shift 0, q_scale 1, on 8 threads, the thread count of the reference's
+    own driver (src/main.c:287)"""
+    from openfish_amd import synth
+    from oracle import crf_oracle as O
+    state_len, T, N, threads = 3, 1666, 16, 8
+    s32 = synth.crf_scores(T, N, state_len, seed=seed, threads=8).astype(np.float32)
+    opt_kw = dict(beam_cut=100.0, blank_score=2.0, q_shift=0.0, q_scale=1.0)
+    if O.have_ref():
+        kind = "reference"
+        run = lambda: O.ref_decode(s32, state_len, opt_kw, nthreads=threads)  # noqa: E731
+    else:
+        kind = "port"
+        run = lambda: O.decode(s32, state_len, opt_kw, nthreads=threads, dump=False)  # noqa: E731
+    run()
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    sec = statistics.median(times)
+    return {"value": round(N / sec, 1), "unit": "chunks/s", "cores": threads, "kind": kind,
+            "sample": "fast: state_len 3, S=64, C=256 fp32, T=1666, N=16, beam 32, beam_cut 100, blank 2.0, q_shift 0, "
+                      "q_scale 1; median of 5 calls of openfish_decode_cpu (%.4f s each)" % sec}
+
+
 def rotary_bench(a):
     """in-place rotary embedding on the shape the reference's driver sketches
     (src/main.c:84-95): batch 500, seqlen 833, 8 heads of 64, rotary_half 32, half data"""
@@ -166,6 +194,8 @@ def main():
     ap.add_argument("--alt-steps", type=int, default=3,
                     help="extra timed calls per side measurement (split scans, hardware-exp scans), reported beside the "
                          "main result (0 = skip)")
+    ap.add_argument("--no-five-columns", action="store_true",
+                    help="skip the side measurement on the same scores with five columns per state (C = 5 * 4^state_len)")
     ap.add_argument("--overlap-steps", type=int, default=5,
                     help="calls per gpubuf of the two-batches-in-flight side measurement (0 = skip)")
     ap.add_argument("--copy-mib", type=int, default=1024,
@@ -190,8 +220,15 @@ def main():
     S = 4 ** state_len
     C = a.columns * S
     scale = synth.stress_scale(N) if stress else None
-    made = synth.crf_scores(T, N, state_len, seed=a.seed, chunk_scale=scale, threads=16, five_columns=a.columns == 5)
-    s16, device_input = (made[0], made[1]) if a.columns == 5 else (made, made)  # s16: the four-column view
+    five_side = a.columns == 4 and a.alt_steps > 0 and not a.no_five_columns
+    made = synth.crf_scores(T, N, state_len, seed=a.seed, chunk_scale=scale, threads=16,
+                            five_columns=a.columns == 5 or five_side)
+    if a.columns == 5:
+        s16, device_input, five = made[0], made[1], None  # s16: the four-column view
+    elif five_side:
+        s16, device_input, five = made[0], made[0], made[1]
+    else:
+        s16, device_input, five = made, made, None
 
     opt = api.DECODER_INIT(q_scale=q_scale, q_shift=q_shift)
     scores = api.upload_scores_to_hip(device_input)
@@ -250,6 +287,21 @@ def main():
                              "scans with v_exp_f32/v_log_f32 only: bwd within 2 ulp, a few posteriors per ten million "
                              "beyond 1e-3 relative; outside the acceptance bar, shown as the memory-bound floor of the kernels")
 
+    # the same scores as the network emits them, five columns per state with a blank first (the layout
+    # BASELINE's configurations name), read in place; its algorithmic bytes count C = 5 * 4^state_len
+    five_columns = None
+    if five is not None:
+        scores5 = api.upload_scores_to_hip(five)
+        del five
+        call5 = (T, N, 5 * S, scores5, state_len, opt)
+        api.openfish_decode_gpu_discard(*call5, gpubuf)
+        ms5, mn5 = timed_decodes(api, gpubuf, call5, a.alt_steps)
+        five_columns = {"C": 5 * S, "chunks_per_s": round(N / (ms5 / 1e3), 1), "ms_per_step": round(ms5, 4),
+                        "stage_ms": {k: round(v, 4) for k, v in mn5.items() if v > 0},
+                        "scan_plus_posterior": scan_stage(algorithmic_bytes(state_len, T, N, 5), mn5),
+                        "note": "the same batch with five fp16 columns per state (blank first, never read), default settings"}
+        scores5.free()
+
     # two batches in flight from one thread: enqueue on one gpubuf while the other one's decode
     # runs (the blocking call is enqueue + wait + copies into fresh host buffers)
     overlap = None
@@ -292,6 +344,7 @@ def main():
 
     opt_kw = dict(beam_cut=100.0, blank_score=2.0, q_shift=q_shift, q_scale=q_scale)
     cpu = cpu_baseline(s16, state_len, opt_kw, min(a.cpu_sample, N)) if a.cpu_sample > 0 else None
+    cpu1 = cpu_baseline_config1(a.seed) if a.cpu_sample > 0 else None
 
     print(json.dumps({
         "metric": "CRF chunks decoded/sec at %s (%d states, T=%d, N=%d); achieved HBM GB/s" % (a.workload, S, T, N),
@@ -305,7 +358,7 @@ def main():
                    "scan_mode": a.scan_mode, "scans": "one kernel" if mean["scan"] > 0 else "two kernels (backward, then forward + posterior beside the beam search)",
                    "seed": a.seed},
         "roofline": roofline, "stages": stages, "other_scan_arrangement": other_split, "fast_scan_mode": fast_mode,
-        "two_in_flight": overlap, "cpu_baseline": cpu,
+        "five_columns": five_columns, "two_in_flight": overlap, "cpu_baseline": cpu, "cpu_baseline_config1": cpu1,
     }))
 
 

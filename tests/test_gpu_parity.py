@@ -433,7 +433,7 @@ def test_constant_scores_closed_form(api):
 FULL = [("fast", 3, 1666, 512, False, 4), ("hac", 4, 1666, 512, False, 4),
         ("sup", 5, 1666, 256, False, 4), ("hac_stress", 4, 1666, 1024, True, 4),
         ("fast_five_columns", 3, 1666, 512, False, 5), ("hac_five_columns", 4, 1666, 512, False, 5),
-        ("sup_five_columns", 5, 1666, 256, False, 5)]
+        ("sup_five_columns", 5, 1666, 256, False, 5), ("hac_stress_five_columns", 4, 1666, 1024, True, 5)]
 
 
 @pytest.mark.parametrize("name,state_len,T,N,stress,columns", FULL)
