@@ -204,11 +204,9 @@ int openfish_amd_last_timings(const openfish_gpubuf_t *gpubuf, float *ms, int n)
  *   the same way, never for real decoding.
  * split scans: 0 (default) runs both scans and the posterior as one kernel, then the beam
  *   search; 1 runs the backward scan, then the forward scan + posterior on a second stream
- *   beside the beam search.  Same results.  Batches whose score tensor has 4 MiB or more per
- *   time step (N * C * 2 bytes) always take the second arrangement: the one-kernel scans lose
- *   half their speed there.  For blocking calls on 64 or 256 states the second arrangement gives
- *   the higher throughput (the forward scan hides beneath the beam search), the first one the
- *   shorter scan stage and the higher throughput with 1024 states.
+ *   beside the beam search.  Same results.  The first arrangement has the shorter scan stage at
+ *   every batch size; the second one hides the forward scan beneath the beam search and can
+ *   come out ahead for blocking calls on small batches.
  */
 void openfish_amd_gpubuf_set_scan_mode(const openfish_gpubuf_t *gpubuf, int scan_mode);
 void openfish_amd_gpubuf_set_split_scans(const openfish_gpubuf_t *gpubuf, int split);

@@ -354,13 +354,7 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
     join_null_stream(g);
     HIP_OK(hipEventRecord(g->ev[EV_START], g->s_main));
     const int cols = columns_of(C, state_len);
-    /* The one-kernel scans walk every chunk from both ends at once.  Once a time step of the score
-     * tensor is 4 MiB or more (2048 chunks of 256 states, 512 of 1024) they fall to half their speed
-     * and below (measured at 256 states: 9.9 ms against 6.2 ms for the split scans at 2048 chunks with
-     * four columns, 9.0 against 8.2 with five, 16.2 against 12.1 at 3072; up to 3.75 MiB they keep
-     * their rate): the split scans take over. */
-    const size_t step_bytes = (size_t)N * (size_t)C * 2;
-    g->pend_split = g->split_scans || step_bytes >= ((size_t)4 << 20);
+    g->pend_split = g->split_scans;
     if (!g->pend_split) {
         /* both sweeps and the posterior in one kernel, then the beam search, all on one stream */
         launch_ok(ofk_scan_posterior(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, cols, stay, g->scan_mode,

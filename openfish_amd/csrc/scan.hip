@@ -1023,6 +1023,18 @@ int states_per_lane(int S, int N, bool backward, int forced) {
 #ifndef OFK_DEPTH_1024
 #define OFK_DEPTH_1024 6
 #endif
+// The one-kernel scans keep the rows of two sweeps in flight.  Rows of one chunk lie N * C * 2 bytes
+// apart; when that is a multiple of 4 MiB (2048 chunks of 256 states, 512 of 1024) all rows in
+// flight fall onto the same DRAM banks, and with sixteen of them (eight per sweep) the kernel ran
+// at half its rate and below (measured, 256 states, 2048 chunks: 8.97 ms; with four rows per sweep
+// 5.69 ms, the rate of smaller batches; at 512 chunks both depths take 1.59 ms).  The separate
+// sweeps, eight rows in flight altogether, never showed it.  Hence half the depth here.
+#ifndef OFK_DEPTH_FUSED
+#define OFK_DEPTH_FUSED 4
+#endif
+#ifndef OFK_DEPTH_FUSED_1024
+#define OFK_DEPTH_FUSED_1024 3
+#endif
 #define OFK_DISPATCH(BACKWARD, LAUNCH, ...)                                                    \
     switch (state_len * 8 + states_per_lane(1 << (2 * state_len), N, BACKWARD, spl)) {        \
         case 3 * 8 + 4: return LAUNCH<64, 4, OFK_DEPTH>(__VA_ARGS__);                          \
@@ -1056,12 +1068,15 @@ static int scan_posterior(const void *scores, float *bwd, float *post, int T, in
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int S = 1 << (2 * state_len);
     switch (state_len * 8 + (state_len >= 3 && state_len <= 5 ? fused_states_per_lane(S, N, spl) : 0)) {
-        case 3 * 8 + 1: return launch_fused<64, 1, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);
-        case 4 * 8 + 4: return launch_fused<256, 4, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);
-        case 4 * 8 + 2: return launch_fused<256, 2, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);
-        case 4 * 8 + 1: return launch_fused<256, 1, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);
-        case 5 * 8 + 4: return launch_fused<1024, 4, OFK_DEPTH_1024>(mode, scores, bwd, post, T, N, stay, st);
-        case 5 * 8 + 2: return launch_fused<1024, 2, OFK_DEPTH_1024>(mode, scores, bwd, post, T, N, stay, st);
+        case 3 * 8 + 1:  // 64 states: latency-bound, the deeper prefetch pays until the rows are 4 MiB apart
+            if ((size_t)N * kCols * S * 2 < ((size_t)4 << 20))
+                return launch_fused<64, 1, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);
+            return launch_fused<64, 1, OFK_DEPTH_FUSED>(mode, scores, bwd, post, T, N, stay, st);
+        case 4 * 8 + 4: return launch_fused<256, 4, OFK_DEPTH_FUSED>(mode, scores, bwd, post, T, N, stay, st);
+        case 4 * 8 + 2: return launch_fused<256, 2, OFK_DEPTH_FUSED>(mode, scores, bwd, post, T, N, stay, st);
+        case 4 * 8 + 1: return launch_fused<256, 1, OFK_DEPTH_FUSED>(mode, scores, bwd, post, T, N, stay, st);
+        case 5 * 8 + 4: return launch_fused<1024, 4, OFK_DEPTH_FUSED_1024>(mode, scores, bwd, post, T, N, stay, st);
+        case 5 * 8 + 2: return launch_fused<1024, 2, OFK_DEPTH_FUSED_1024>(mode, scores, bwd, post, T, N, stay, st);
         default: return OFK_BAD_ARGS;
     }
 }
