@@ -116,7 +116,7 @@ void openfish_amd_lse_table(double *out) { build_lse_table(out); }
 
 #define OFA_MAGIC 0x6f66616d64677075ull /* "ofamdgpu" */
 
-enum { EV_JOIN, EV_START, EV_BWD_END, EV_BEAM_START, EV_BEAM_END, EV_FWD_END, EV_SEQ_START, EV_SEQ_END, EV_COUNT };
+enum { EV_JOIN, EV_START, EV_BWD_END, EV_BEAM_START, EV_BEAM_END, EV_FWD_END, EV_SEQ_START, EV_SEQ_END, EV_SEQ_COPIED, EV_COUNT };
 /* with both sweeps in one kernel EV_BWD_END marks its end and EV_FWD_END is not recorded */
 
 typedef struct {
@@ -398,6 +398,7 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
                            state_len, phred_for(g, options), g->s_main), "sequence");
     HIP_OK(hipEventRecord(g->ev[EV_SEQ_END], g->s_main));
     HIP_OK(hipMemcpyAsync(g->h_out + nt, g->pub.sequence, nt, hipMemcpyDeviceToHost, g->s_main));
+    HIP_OK(hipEventRecord(g->ev[EV_SEQ_COPIED], g->s_main)); /* the host takes the bases while the qualities travel */
     HIP_OK(hipMemcpyAsync(g->h_out + 2 * nt, g->pub.qstring, nt, hipMemcpyDeviceToHost, g->s_main));
     g->pending = 1;
     g->pend_T = T;
@@ -417,8 +418,9 @@ void openfish_decode_gpu(const int T, const int N, const int C, void *scores_TNC
     alloc_outputs(T, N, moves, sequence, qstring);
     HIP_OK(hipStreamSynchronize(g->s_side));
     memcpy(*moves, g->h_out, nt);
-    HIP_OK(hipStreamSynchronize(g->s_main));
+    HIP_OK(hipEventSynchronize(g->ev[EV_SEQ_COPIED]));
     memcpy(*sequence, g->h_out + nt, nt);
+    HIP_OK(hipStreamSynchronize(g->s_main));
     memcpy(*qstring, g->h_out + 2 * nt, nt);
     g->pending = 0;
     g->timed = 1;
