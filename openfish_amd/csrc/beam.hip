@@ -173,7 +173,12 @@ __device__ __forceinline__ int wave_sum_i(int x) {
 }
 __device__ __forceinline__ uint64_t ballot(bool p) { return __builtin_amdgcn_ballot_w64(p); }
 // per lane: yes where the lane's bit of a wave-wide mask is set, no elsewhere; the mask goes into
-// the select as it is (a comparison result the wave already holds in scalar registers)
+// the select as it is (a comparison result the wave already holds in scalar registers).
+// The compiler cannot see into these two statements, so it inserts no wait states for them.  None
+// are due: a scalar pair written by a vector comparison may be read as the mask of a select or as
+// a carry by the next vector instruction (the wait states the architecture asks for after such a
+// write concern lane selects of v_readlane/v_writelane, v_div_fmas and memory instructions).  A
+// mask that is to be read by v_readlane or as an address goes through an s_mov first.
 __device__ __forceinline__ int pick_by_bit(uint64_t mask, int yes, int no) {
     int r;
     asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(no), "v"(yes), "s"(mask));

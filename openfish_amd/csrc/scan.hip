@@ -252,11 +252,18 @@ __device__ __forceinline__ float add_half(uint32_t word, float x) {
 // A state's scores are kCols consecutive fp16 values: the four transitions, after kLead
 // values that the decoder never reads (the blank column of five-column scores).  With
 // four columns a lane's window is contiguous and is fetched with vector loads; with five
-// it is fetched two bytes at a time, straight from the caller's layout.
+// it is fetched straight from the caller's layout, 32 bits at a time where two wanted values
+// are neighbours (from addresses that are only 2-byte aligned, which global loads accept), two
+// bytes at a time elsewhere.
 __device__ __forceinline__ uint32_t half_at(const _Float16 *p) { return *reinterpret_cast<const uint16_t *>(p); }
 __device__ __forceinline__ uint32_t half_pair_at(const _Float16 *p) {
-    if constexpr (kCols == 4) return *reinterpret_cast<const uint32_t *>(p);
-    else return half_at(p) | (half_at(p + 1) << 16);
+    if constexpr (kCols == 4) {
+        return *reinterpret_cast<const uint32_t *>(p);
+    } else {  // one 32-bit load from an address that is only 2-byte aligned
+        uint32_t w;
+        __builtin_memcpy(&w, p, 4);
+        return w;
+    }
 }
 
 // Backward: transition b of own state i is element kCols * b + i of the lane's window
@@ -935,6 +942,11 @@ __global__ __launch_bounds__((FusedShape<S, SPL>::kThreads), 4) void scan_post_k
 
 const LogSeries kSeries = {OFA_LOG_SERIES, OFA_EXP_COEFS};
 
+// The always-double and the hardware-only arithmetic exist for tests and measurements: they are
+// built with the fewest states per lane only (the entry points below ask for nothing else).
+template <int S>
+constexpr int kPlainSpl = S >= 1024 ? 2 : 1;
+
 template <int S, int SPL, int DEPTH>
 int launch_bwd(int mode, const void *scores, float *bwd, int T, int N, float stay, hipStream_t st) {
     using Sh = Shape<S, SPL>;
@@ -945,10 +957,16 @@ int launch_bwd(int mode, const void *scores, float *bwd, int T, int N, float sta
             hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, OFK_SCAN_TWO_TIER>), grid, block, 0, st, sc, bwd, T, N, stay, kSeries);
             break;
         case OFK_SCAN_PRECISE:
-            hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, OFK_SCAN_PRECISE>), grid, block, 0, st, sc, bwd, T, N, stay, kSeries);
+            if constexpr (SPL == kPlainSpl<S>)
+                hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, OFK_SCAN_PRECISE>), grid, block, 0, st, sc, bwd, T, N, stay, kSeries);
+            else
+                return OFK_BAD_ARGS;
             break;
         case OFK_SCAN_FAST:
-            hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, OFK_SCAN_FAST>), grid, block, 0, st, sc, bwd, T, N, stay, kSeries);
+            if constexpr (SPL == kPlainSpl<S>)
+                hipLaunchKernelGGL((bwd_scan_kernel<S, SPL, DEPTH, OFK_SCAN_FAST>), grid, block, 0, st, sc, bwd, T, N, stay, kSeries);
+            else
+                return OFK_BAD_ARGS;
             break;
         default: return OFK_BAD_ARGS;
     }
@@ -965,10 +983,16 @@ int launch_fwd(int mode, const void *scores, const float *bwd, float *post, int 
             hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, OFK_SCAN_TWO_TIER>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
             break;
         case OFK_SCAN_PRECISE:
-            hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, OFK_SCAN_PRECISE>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            if constexpr (SPL == kPlainSpl<S>)
+                hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, OFK_SCAN_PRECISE>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            else
+                return OFK_BAD_ARGS;
             break;
         case OFK_SCAN_FAST:
-            hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, OFK_SCAN_FAST>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            if constexpr (SPL == kPlainSpl<S>)
+                hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, OFK_SCAN_FAST>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            else
+                return OFK_BAD_ARGS;
             break;
         default: return OFK_BAD_ARGS;
     }
@@ -985,10 +1009,16 @@ int launch_fused(int mode, const void *scores, float *bwd, float *post, int T, i
             hipLaunchKernelGGL((scan_post_kernel<S, SPL, DEPTH, OFK_SCAN_TWO_TIER>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
             break;
         case OFK_SCAN_PRECISE:
-            hipLaunchKernelGGL((scan_post_kernel<S, SPL, DEPTH, OFK_SCAN_PRECISE>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            if constexpr (SPL == kPlainSpl<S>)
+                hipLaunchKernelGGL((scan_post_kernel<S, SPL, DEPTH, OFK_SCAN_PRECISE>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            else
+                return OFK_BAD_ARGS;
             break;
         case OFK_SCAN_FAST:
-            hipLaunchKernelGGL((scan_post_kernel<S, SPL, DEPTH, OFK_SCAN_FAST>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            if constexpr (SPL == kPlainSpl<S>)
+                hipLaunchKernelGGL((scan_post_kernel<S, SPL, DEPTH, OFK_SCAN_FAST>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
+            else
+                return OFK_BAD_ARGS;
             break;
         default: return OFK_BAD_ARGS;
     }
@@ -1036,7 +1066,7 @@ int states_per_lane(int S, int N, bool backward, int forced) {
 #define OFK_DEPTH_FUSED_1024 3
 #endif
 #define OFK_DISPATCH(BACKWARD, LAUNCH, ...)                                                    \
-    switch (state_len * 8 + states_per_lane(1 << (2 * state_len), N, BACKWARD, spl)) {        \
+    switch (state_len * 8 + states_per_lane(1 << (2 * state_len), N, BACKWARD, lanes_asked(mode, spl))) { \
         case 3 * 8 + 4: return LAUNCH<64, 4, OFK_DEPTH>(__VA_ARGS__);                          \
         case 3 * 8 + 2: return LAUNCH<64, 2, OFK_DEPTH>(__VA_ARGS__);                          \
         case 3 * 8 + 1: return LAUNCH<64, 1, OFK_DEPTH>(__VA_ARGS__);                          \
@@ -1061,13 +1091,16 @@ static int fused_states_per_lane(int S, int N, int forced) {
     return min_spl;
 }
 
+// states per lane to force: the caller's wish (0 = none) with the default arithmetic, the fewest otherwise
+static int lanes_asked(int mode, int spl) { return mode == OFK_SCAN_TWO_TIER ? spl : 1; }
+
 static int scan_posterior(const void *scores, float *bwd, float *post, int T, int N, int state_len, float stay,
                           int mode, int spl, void *stream) {
     if (!scores || !bwd || !post || T < 1 || N < 1 || !aligned16(scores) || !aligned16(bwd) || !aligned16(post))
         return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int S = 1 << (2 * state_len);
-    switch (state_len * 8 + (state_len >= 3 && state_len <= 5 ? fused_states_per_lane(S, N, spl) : 0)) {
+    switch (state_len * 8 + (state_len >= 3 && state_len <= 5 ? fused_states_per_lane(S, N, lanes_asked(mode, spl)) : 0)) {
         case 3 * 8 + 1:  // 64 states: latency-bound, the deeper prefetch pays until the rows are 4 MiB apart
             if ((size_t)N * kCols * S * 2 < ((size_t)4 << 20))
                 return launch_fused<64, 1, OFK_DEPTH>(mode, scores, bwd, post, T, N, stay, st);

@@ -108,7 +108,9 @@ def test_every_states_per_lane_choice_gives_the_oracle_s_tensors(api, state_len,
     """states per lane forced through the gpubuf's setter (the automatic choice depends on the batch
     size and never reaches most of them at test sizes), on small uneven batches, in both scan
     arrangements: bwd bit-identical to the oracle, the posterior within 1e-3, and the default
-    arithmetic bit-identical to the always-double one"""
+    arithmetic bit-identical to the always-double one (which is built with the fewest states per
+    lane only and ignores the setter: the posteriors, whose normalising sum is taken in an order
+    that depends on the lanes, are compared bit for bit where both ran with the same number)"""
     S = 4 ** state_len
     s16 = synth.crf_scores(T, N, state_len, seed=31 * spl + T, chunk_scale=synth.stress_scale(N) if state_len == 4 else None)
     ref_bwd, _, ref_post = O.scans(s16.astype(np.float32), state_len)
@@ -123,4 +125,7 @@ def test_every_states_per_lane_choice_gives_the_oracle_s_tensors(api, state_len,
         assert np.array_equal(gb.tensor("bwd_NTC"), ref_bwd), mode
         posts[mode] = gb.tensor("post_NTC")
         close(posts[mode], ref_post)
-    assert np.array_equal(posts["two_tier"], posts["precise"])
+    fewest = 2 if state_len == 5 else 1
+    used = max(spl, fewest) if (split or state_len != 3) else 1  # one kernel, 64 states: always one state per lane
+    if used == fewest:
+        assert np.array_equal(posts["two_tier"], posts["precise"])
