@@ -179,8 +179,8 @@ def scan_stage(need, mean):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="hac", choices=sorted(WORKLOADS) + ["rotary"])
     ap.add_argument("--chunks", type=int, default=0, help="override N")
     ap.add_argument("--columns", type=int, default=4, choices=(4, 5),
