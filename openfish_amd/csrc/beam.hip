@@ -1009,7 +1009,7 @@ int launch_beam(const void *scores, const float *bwd, ofk_beam_slot_t *beam, int
     // 256 compute units: up to 512 chunks fit two to a unit; larger batches go four to a group
     // where the LDS of four chunks fits (64 and 256 states)
     if constexpr (S <= 256) {
-        if (N > 512) {
+        if (N > OFK_SPARSE_SEARCH_MAX_CHUNKS) {
             hipLaunchKernelGGL((beam_kernel<S, 4, COLS>), dim3((N + 3) / 4), dim3(512), 0, st,
                                static_cast<const _Float16 *>(scores), bwd, beam, states, moves, T, N, log_cut,
                                stay, flags, lse_table);

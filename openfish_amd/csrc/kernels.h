@@ -80,9 +80,19 @@ typedef struct {
     float thr[OFK_PHRED_STEPS];
 } ofk_phred_table_t;
 
+/* path_sums: NULL, or what ofk_path_sums left for these posteriors (post is then not read). */
 int ofk_sequence(const float *post, int32_t *states, const uint8_t *moves, float *qual_data,
                  float *base_probs, float *total_probs, char *sequence, char *qstring, int T, int N,
-                 int state_len, const ofk_phred_table_t *phred, void *stream);
+                 int state_len, const ofk_phred_table_t *phred, const float *path_sums, void *stream);
+/* sums[n][t][s], N x T x states floats: posterior of state s at row t + 1 of chunk n plus that of its
+ * distinct one-base shifts, fp32 sums in the CPU path's order (src/beam_search.c:441-463), for every
+ * state: the input of a block's quality whichever state the path then takes. */
+int ofk_path_sums(const float *post, float *sums, int T, int N, int state_len, void *stream);
+/* Batches up to this size put at most two chunks of the beam search on a compute unit (one wave
+ * each): the search then leaves room for ofk_path_sums beside it.  Larger batches fill the units
+ * with search waves, and the extra kernel was measured to cost the search more than it saves the
+ * sequence stage (1024 chunks of 256 states: search 1.42 -> 1.77 ms, sequence 0.32 -> 0.13 ms). */
+#define OFK_SPARSE_SEARCH_MAX_CHUNKS 512
 /* device-to-device copy of `bytes` (a multiple of 16); the calibration kernel for counters */
 int ofk_copy(void *dst, const void *src, size_t bytes, void *stream);
 int ofk_rotary_emb(void *x, const float *sin_buf, const float *cos_buf, int batch, int seqlen,

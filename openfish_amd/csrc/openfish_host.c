@@ -116,7 +116,7 @@ void openfish_amd_lse_table(double *out) { build_lse_table(out); }
 
 #define OFA_MAGIC 0x6f66616d64677075ull /* "ofamdgpu" */
 
-enum { EV_JOIN, EV_START, EV_BWD_END, EV_BEAM_START, EV_BEAM_END, EV_FWD_END, EV_SEQ_START, EV_SEQ_END, EV_COUNT };
+enum { EV_JOIN, EV_START, EV_BWD_END, EV_BEAM_START, EV_BEAM_END, EV_FWD_END, EV_SEQ_START, EV_SEQ_END, EV_SUMS_END, EV_COUNT };
 /* with both sweeps in one kernel EV_BWD_END marks its end and EV_FWD_END is not recorded */
 
 typedef struct {
@@ -124,6 +124,7 @@ typedef struct {
     unsigned long long magic;
     int T, N, state_len;
     void *slab;            /* one device allocation behind all pub fields */
+    float *path_sums;      /* N x T x states: per state, the posteriors a block's quality is made of, summed */
     unsigned char *h_out;  /* pinned host memory for moves | sequence | qstring */
     unsigned char *d_out;  /* the same memory as the device addresses it */
     double *lse_table;     /* device copy of the log(1 + e^-gap) table */
@@ -166,19 +167,21 @@ openfish_gpubuf_t *openfish_gpubuf_init(const int T, const int N, const int stat
 
     /* field sizes as in the reference (src/decode_hip.hip:24-48) except beam_vector,
      * whose slots are 2 bytes here */
-    const size_t sz[10] = {tens, tens, nt, nt, nt,
+    const size_t sz[11] = {tens, tens, nt, nt, nt,
                            sizeof(ofk_beam_slot_t) * (size_t)N * OFK_BEAM_WIDTH * (size_t)(T + 1),
-                           sizeof(int32_t) * nt, sizeof(float) * 4 * nt, sizeof(float) * nt, sizeof(float) * nt};
+                           sizeof(int32_t) * nt, sizeof(float) * 4 * nt, sizeof(float) * nt, sizeof(float) * nt,
+                           /* path_sums, not a field of the reference's struct; see enqueue_decode */
+                           (state_len <= 4 ? sizeof(float) * S * (size_t)T * (size_t)(N < OFK_SPARSE_SEARCH_MAX_CHUNKS ? N : OFK_SPARSE_SEARCH_MAX_CHUNKS) : 0)};
     size_t total = 0;
-    for (int i = 0; i < 10; ++i) total += round_up(sz[i]);
+    for (int i = 0; i < 11; ++i) total += round_up(sz[i]);
     HIP_OK(hipMalloc(&g->slab, total));
     unsigned char *p = (unsigned char *)g->slab;
-    void **field[10] = {(void **)&g->pub.bwd_NTC, (void **)&g->pub.post_NTC, (void **)&g->pub.moves,
+    void **field[11] = {(void **)&g->pub.bwd_NTC, (void **)&g->pub.post_NTC, (void **)&g->pub.moves,
                         (void **)&g->pub.sequence, (void **)&g->pub.qstring, &g->pub.beam_vector,
                         &g->pub.states, (void **)&g->pub.qual_data, (void **)&g->pub.base_probs,
-                        (void **)&g->pub.total_probs};
-    for (int i = 0; i < 10; ++i) {
-        *field[i] = p;
+                        (void **)&g->pub.total_probs, (void **)&g->path_sums};
+    for (int i = 0; i < 11; ++i) {
+        *field[i] = sz[i] ? p : NULL;
         p += round_up(sz[i]);
     }
     HIP_OK(hipHostMalloc((void **)&g->h_out, 3 * nt, hipHostMallocDefault));
@@ -357,6 +360,9 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
     HIP_OK(hipEventRecord(g->ev[EV_START], g->s_main));
     const int cols = columns_of(C, state_len);
     g->pend_split = g->split_scans;
+    /* only where the search leaves the machine idle, and not with 1024 states, whose search waits for
+     * memory and was measured to take half as long again beside the extra kernel */
+    const int use_sums = !g->pend_split && g->path_sums != NULL && N <= OFK_SPARSE_SEARCH_MAX_CHUNKS;
     if (!g->pend_split) {
         /* both sweeps and the posterior in one kernel, then the beam search, all on one stream */
         launch_ok(ofk_scan_posterior(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, cols, stay, g->scan_mode,
@@ -367,9 +373,18 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
                                   (int32_t *)g->pub.states, g->pub.moves, T, N, state_len, cols, log_beam_cut(options),
                                   stay, g->lse_table, g->debug_flags, g->s_main), "beam_search");
         HIP_OK(hipEventRecord(g->ev[EV_BEAM_END], g->s_main));
+        /* The search keeps one wave per chunk busy and leaves the rest of the machine idle: beside
+         * it, on the second stream, the posteriors that a block's quality is made of are summed for
+         * every state, so that the sequence stage reads one value per time step instead of nine. */
+        if (use_sums) {
+            HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BWD_END], 0));
+            launch_ok(ofk_path_sums(g->pub.post_NTC, g->path_sums, T, N, state_len, g->s_side), "path_sums");
+            HIP_OK(hipEventRecord(g->ev[EV_SUMS_END], g->s_side));
+        }
         /* the moves are final once the beam search is: they travel while the sequence stage runs */
         HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BEAM_END], 0));
         HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_side));
+        if (use_sums) HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_SUMS_END], 0));
     } else {
         launch_ok(ofk_bwd_scan(scores_TNC, g->pub.bwd_NTC, T, N, state_len, cols, stay, g->scan_mode, g->scan_spl, g->s_main),
                   "bwd_scan");
@@ -402,7 +417,7 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
      * are filled by the stage-level entry points only. */
     launch_ok(ofk_sequence(g->pub.post_NTC, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data,
                            g->pub.base_probs, g->pub.total_probs, (char *)g->d_out + nt, (char *)g->d_out + 2 * nt, T, N,
-                           state_len, phred_for(g, options), g->s_main), "sequence");
+                           state_len, phred_for(g, options), use_sums ? g->path_sums : NULL, g->s_main), "sequence");
     HIP_OK(hipEventRecord(g->ev[EV_SEQ_END], g->s_main));
     g->pending = 1;
     g->pend_T = T;
@@ -555,7 +570,7 @@ void openfish_amd_sequence(int T, int N, int state_len, const openfish_opt_t *op
     ofa_gpubuf_t *g = checked(gpubuf, T, N, state_len);
     launch_ok(ofk_sequence(post, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data, g->pub.base_probs,
                            g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N, state_len,
-                           phred_for(g, options), NULL), "sequence");
+                           phred_for(g, options), NULL, NULL), "sequence");
     HIP_OK(hipStreamSynchronize(0));
 }
 
@@ -573,7 +588,7 @@ void openfish_amd_decode_from_tensors(int T, int N, int C, const void *scores, i
                               g->lse_table, g->debug_flags, g->s_main), "beam_search");
     launch_ok(ofk_sequence(post, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data, g->pub.base_probs,
                            g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N, state_len,
-                           phred_for(g, options), g->s_main), "sequence");
+                           phred_for(g, options), NULL, g->s_main), "sequence");
     fetch_outputs(g, T, N, moves, sequence, qstring);
 }
 

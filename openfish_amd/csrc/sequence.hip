@@ -23,7 +23,8 @@ template <int S>
 __global__ __launch_bounds__(kThreads) void sequence_kernel(
     const float *__restrict__ post, int32_t *__restrict__ states, const uint8_t *__restrict__ moves,
     float *__restrict__ qual_data, float *__restrict__ base_probs, float *__restrict__ total_probs,
-    char *__restrict__ sequence, char *__restrict__ qstring, int T, ofk_phred_table_t phred) {
+    char *__restrict__ sequence, char *__restrict__ qstring, int T, ofk_phred_table_t phred,
+    const float *__restrict__ path_sums) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     float *s_prob = reinterpret_cast<float *>(lds);        // [T] called-base probability
     float *s_wrong = s_prob + T;                           // [T] probability of each other base
@@ -43,20 +44,25 @@ __global__ __launch_bounds__(kThreads) void sequence_kernel(
         const int st = st_n[t];
         const int base = st & 3;
         st_n[t] = base;
-        const float *p = post_n + (size_t)(t + 1) * S;
-        float prob = p[st];
-        int nb[8];
+        float prob;
+        if (path_sums) {  // the sum below, taken for every state by path_sums_kernel: one read instead of nine
+            prob = path_sums[((size_t)n * T + t) * S + st];
+        } else {
+            const float *p = post_n + (size_t)(t + 1) * S;
+            prob = p[st];
+            int nb[8];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            nb[2 * b] = (st >> 2) + (S / 4) * b;
-            nb[2 * b + 1] = ((st << 2) & (S - 1)) + b;
-        }
+            for (int b = 0; b < 4; ++b) {
+                nb[2 * b] = (st >> 2) + (S / 4) * b;
+                nb[2 * b + 1] = ((st << 2) & (S - 1)) + b;
+            }
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            bool fresh = nb[k] != st;
+            for (int k = 0; k < 8; ++k) {
+                bool fresh = nb[k] != st;
 #pragma unroll
-            for (int m = 0; m < k; ++m) fresh = fresh && nb[m] != nb[k];
-            if (fresh) prob += p[nb[k]];
+                for (int m = 0; m < k; ++m) fresh = fresh && nb[m] != nb[k];
+                if (fresh) prob += p[nb[k]];
+            }
         }
         if (prob > 1.0f) prob = 1.0f;
         else if (prob < 0.0f) prob = 0.0f;
@@ -132,10 +138,132 @@ __global__ __launch_bounds__(kThreads) void sequence_kernel(
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// For every chunk, time step and state: the posterior of the k-mer plus that of its distinct
+// one-base shifts, summed in the CPU path's order -- what step 1 of sequence_kernel gathers for
+// the one state on the path.  Those nine scattered reads per time step fetch about half of the
+// posteriors, 64 bytes for every 4 wanted, and made up most of that kernel's time; they come
+// after the beam search, which leaves most of the machine idle for a millisecond.  This kernel
+// runs beside the search, reads every row once, in order, and the sequence stage then takes one
+// value per time step.
+//
+// A wave owns whole rows (four at a time with 64 states) and keeps the current one in LDS, 256
+// floats per 64 lanes; lane j holds states 4j .. 4j+3 of each 256.  Those four share their
+// four predecessors (st >> 2) + b * S/4, and the successors 4 * (st mod S/4) + b of a state are
+// four neighbours in the row: eight LDS reads per lane cover all 32 values.  Which of a state's
+// eight neighbours count (not the state itself, not an earlier neighbour) does not depend on
+// the time step and is worked out once per lane.  A wave's LDS operations complete in order, so
+// the waves of a group never wait for each other.
+// ---------------------------------------------------------------------------------------------
+template <int S>
+__global__ __launch_bounds__(256) void path_sums_kernel(const float *__restrict__ post, float *__restrict__ sums,
+                                                        int T, long rows) {
+    constexpr int Q = S / 4;
+    constexpr int G = S >= 256 ? S / 256 : 1;       // float4 pieces of a row per lane
+    constexpr int kRowsPerTile = S >= 256 ? 1 : 4;  // rows a wave takes at a time
+    constexpr int kTile = S >= 256 ? S : 256;       // floats
+    __shared__ __attribute__((aligned(16))) float tiles[4][kTile];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float *tile = tiles[wave];
+    const int sub = S >= 256 ? 0 : lane >> 4;           // row of the tile this lane works on
+    const int j0 = S >= 256 ? lane : lane & 15;         // quad of states within 256 (within the row, with 64 states)
+    float *row = tile + (S >= 256 ? 0 : 64 * sub);      // this lane's row in LDS
+
+    // per state: which neighbours are added (bit k: neighbour k, predecessors at even k)
+    uint32_t fresh[G][4];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int st = 4 * (j0 + 64 * g) + i;
+            int nb[8];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                nb[2 * b] = (st >> 2) + Q * b;
+                nb[2 * b + 1] = ((st << 2) & (S - 1)) + b;
+            }
+            uint32_t bits = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                bool f = nb[k] != st;
+#pragma unroll
+                for (int m = 0; m < k; ++m) f = f && nb[m] != nb[k];
+                bits |= f ? 1u << k : 0u;
+            }
+            fresh[g][i] = bits;
+        }
+    }
+
+    const long tiles_n = (rows + kRowsPerTile - 1) / kRowsPerTile;
+    const long step = (long)gridDim.x * 4;
+    long tix = (long)blockIdx.x * 4 + wave;
+    // row r of the output is time step r % T of chunk r / T and reads row r % T + 1 of that chunk's posteriors
+    auto in_row = [&](long r) { return post + ((size_t)(r / T) * (size_t)(T + 1) + (size_t)(r % T) + 1) * S; };
+    float4 cur[G], nxt[G];
+    auto fetch = [&](long t_ix, float4 (&v)[G]) {
+        const long r = t_ix * kRowsPerTile + sub;
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+            v[g] = (t_ix < tiles_n && r < rows) ? *reinterpret_cast<const float4 *>(in_row(r) + 4 * (j0 + 64 * g))
+                                                : make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    fetch(tix, cur);
+    for (; tix < tiles_n; tix += step) {
+        fetch(tix + step, nxt);
+#pragma unroll
+        for (int g = 0; g < G; ++g) *reinterpret_cast<float4 *>(row + 4 * (j0 + 64 * g)) = cur[g];
+        __builtin_amdgcn_wave_barrier();
+        const long r = tix * kRowsPerTile + sub;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int j = j0 + 64 * g;  // the lane's states 4j .. 4j+3 share their predecessors j + b * Q
+            float prev[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) prev[b] = row[j + Q * b];
+            const float own[4] = {cur[g].x, cur[g].y, cur[g].z, cur[g].w};
+            float out[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int st = 4 * j + i;
+                const float4 nx = *reinterpret_cast<const float4 *>(row + 4 * (st & (Q - 1)));
+                const float next[4] = {nx.x, nx.y, nx.z, nx.w};
+                float prob = own[i];  // fp32 sums in the CPU path's order
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const float with_prev = prob + prev[b];
+                    prob = (fresh[g][i] >> (2 * b)) & 1u ? with_prev : prob;
+                    const float with_next = prob + next[b];
+                    prob = (fresh[g][i] >> (2 * b + 1)) & 1u ? with_next : prob;
+                }
+                out[i] = prob;
+            }
+            if (r < rows)
+                *reinterpret_cast<float4 *>(sums + (size_t)r * S + 4 * j) = make_float4(out[0], out[1], out[2], out[3]);
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int g = 0; g < G; ++g) cur[g] = nxt[g];
+    }
+}
+
+template <int S>
+int launch_path_sums(const float *post, float *sums, int T, int N, hipStream_t st) {
+    const long rows = (long)N * T;
+    // Half as many workgroups as chunks, up to one per compute unit (one wave per SIMD): with 512
+    // chunks of 256 states the kernel then ends well inside the beam search it runs beside and does
+    // not slow it (measured: 256 groups 1.185 ms of search against 1.183 alone, 512 groups 1.195,
+    // 1024 groups 1.27; 128 groups outlast the search).
+    int wgs = N / 2;
+    wgs = wgs < 64 ? 64 : (wgs > 256 ? 256 : wgs);
+    hipLaunchKernelGGL((path_sums_kernel<S>), dim3(wgs), dim3(256), 0, st, post, sums, T, rows);
+    return (int)hipGetLastError();
+}
+
 template <int S>
 int launch_sequence(const float *post, int32_t *states, const uint8_t *moves, float *qual_data,
                     float *base_probs, float *total_probs, char *sequence, char *qstring, int T, int N,
-                    const ofk_phred_table_t &phred, hipStream_t st) {
+                    const ofk_phred_table_t &phred, const float *path_sums, hipStream_t st) {
     const size_t lds = (size_t)T * (4 + 4 + 1 + 1) + (size_t)(T + 1) * 4;
     if (lds > 64 * 1024) {  // beyond the default limit of dynamic LDS; the compute unit has 160 KB
         const hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void *>(&sequence_kernel<S>),
@@ -143,25 +271,37 @@ int launch_sequence(const float *post, int32_t *states, const uint8_t *moves, fl
         if (rc != hipSuccess) return (int)rc;
     }
     hipLaunchKernelGGL((sequence_kernel<S>), dim3(N), dim3(kThreads), lds, st, post, states, moves, qual_data,
-                       base_probs, total_probs, sequence, qstring, T, phred);
+                       base_probs, total_probs, sequence, qstring, T, phred, path_sums);
     return (int)hipGetLastError();
 }
 
 }  // namespace
 
+extern "C" int ofk_path_sums(const float *post, float *sums, int T, int N, int state_len, void *stream) {
+    if (!post || !sums || T < 1 || N < 1) return OFK_BAD_ARGS;
+    if ((reinterpret_cast<uintptr_t>(post) | reinterpret_cast<uintptr_t>(sums)) & 15u) return OFK_BAD_ARGS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (state_len) {
+        case 3: return launch_path_sums<64>(post, sums, T, N, st);
+        case 4: return launch_path_sums<256>(post, sums, T, N, st);
+        case 5: return launch_path_sums<1024>(post, sums, T, N, st);
+        default: return OFK_BAD_ARGS;
+    }
+}
+
 extern "C" int ofk_sequence(const float *post, int32_t *states, const uint8_t *moves, float *qual_data,
                             float *base_probs, float *total_probs, char *sequence, char *qstring, int T, int N,
-                            int state_len, const ofk_phred_table_t *phred, void *stream) {
+                            int state_len, const ofk_phred_table_t *phred, const float *path_sums, void *stream) {
     // the per-chunk tables live in LDS: 14 bytes per time step
-    if (!post || !states || !moves || !qual_data || !base_probs || !total_probs || !sequence || !qstring ||
+    if ((!post && !path_sums) || !states || !moves || !qual_data || !base_probs || !total_probs || !sequence || !qstring ||
         !phred || T < 1 || T > OFK_MAX_T || N < 1)
         return OFK_BAD_ARGS;
     if (reinterpret_cast<uintptr_t>(qual_data) & 15u) return OFK_BAD_ARGS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (state_len) {
-        case 3: return launch_sequence<64>(post, states, moves, qual_data, base_probs, total_probs, sequence, qstring, T, N, *phred, st);
-        case 4: return launch_sequence<256>(post, states, moves, qual_data, base_probs, total_probs, sequence, qstring, T, N, *phred, st);
-        case 5: return launch_sequence<1024>(post, states, moves, qual_data, base_probs, total_probs, sequence, qstring, T, N, *phred, st);
+        case 3: return launch_sequence<64>(post, states, moves, qual_data, base_probs, total_probs, sequence, qstring, T, N, *phred, path_sums, st);
+        case 4: return launch_sequence<256>(post, states, moves, qual_data, base_probs, total_probs, sequence, qstring, T, N, *phred, path_sums, st);
+        case 5: return launch_sequence<1024>(post, states, moves, qual_data, base_probs, total_probs, sequence, qstring, T, N, *phred, path_sums, st);
         default: return OFK_BAD_ARGS;
     }
 }
