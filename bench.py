@@ -63,6 +63,7 @@ def algorithmic_bytes(state_len, T, N, columns=4):
         "fwd_post": N * (scores + 2 * vec),           # read scores + bwd, write post
         "beam": N * (scores + T * S * 4 + (T + 1) * 32 * 2 * 2 + 5 * T),  # rows, beam slots out+in, states+moves
         "sequence": N * (9 * 4 * T + 5 * T + 16 * T + 8 * T + 2 * T),  # gathers, states/moves, qual, probs, text
+        "path_sums": N * 2 * T * S * 4,               # read the posteriors of T rows, write a sum per state
     }
     need["scan"] = need["bwd"] + need["fwd_post"]     # both scans + posterior as one kernel: the same minimum
     return need
@@ -252,7 +253,7 @@ def main():
 
     need = algorithmic_bytes(state_len, T, N, a.columns)
     stages = {}
-    for k in ("scan", "bwd", "fwd_post", "beam", "sequence"):
+    for k in ("scan", "bwd", "fwd_post", "beam", "sequence", "path_sums"):  # path_sums runs beside the beam search
         if mean[k] > 0:
             stages[k] = {"ms": round(mean[k], 4), "algorithmic_GB": round(need[k] / 1e9, 4),
                          "GBps": round(need[k] / 1e9 / (mean[k] / 1e3), 1)}

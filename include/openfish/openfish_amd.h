@@ -176,7 +176,9 @@ enum openfish_amd_stage {
     OPENFISH_AMD_STAGE_SEQ = 3,   /* quality + sequence kernel */
     OPENFISH_AMD_STAGE_TOTAL = 4, /* first launch to last kernel end, device side */
     OPENFISH_AMD_STAGE_SCAN = 5,  /* both scans + posterior as one kernel (0 when they ran split) */
-    OPENFISH_AMD_STAGE_COUNT = 6
+    OPENFISH_AMD_STAGE_SUMS = 6,  /* per-state sums of posteriors for the quality stage, a kernel that runs beside the
+                                   * beam search on a second stream (0 when the decode did without it) */
+    OPENFISH_AMD_STAGE_COUNT = 7
 };
 
 /*

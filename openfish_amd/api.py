@@ -22,7 +22,7 @@ if not os.path.exists(LIB_PATH):
 
 _L = C.CDLL(LIB_PATH)
 
-STAGES = ("bwd", "fwd_post", "beam", "sequence", "total", "scan")
+STAGES = ("bwd", "fwd_post", "beam", "sequence", "total", "scan", "path_sums")
 # enum openfish_amd_scan_mode
 SCAN_TWO_TIER, SCAN_PRECISE, SCAN_FAST = 0, 1, 2
 SCAN_MODES = {"two_tier": SCAN_TWO_TIER, "precise": SCAN_PRECISE, "fast": SCAN_FAST}

@@ -116,7 +116,7 @@ void openfish_amd_lse_table(double *out) { build_lse_table(out); }
 
 #define OFA_MAGIC 0x6f66616d64677075ull /* "ofamdgpu" */
 
-enum { EV_JOIN, EV_START, EV_BWD_END, EV_BEAM_START, EV_BEAM_END, EV_FWD_END, EV_SEQ_START, EV_SEQ_END, EV_SUMS_END, EV_COUNT };
+enum { EV_JOIN, EV_START, EV_BWD_END, EV_BEAM_START, EV_BEAM_END, EV_FWD_END, EV_SEQ_START, EV_SEQ_END, EV_SUMS_START, EV_SUMS_END, EV_COUNT };
 /* with both sweeps in one kernel EV_BWD_END marks its end and EV_FWD_END is not recorded */
 
 typedef struct {
@@ -133,7 +133,7 @@ typedef struct {
     float ms[OPENFISH_AMD_STAGE_COUNT];
     int timed;
     int pending;           /* a decode has been enqueued and not yet waited for */
-    int pend_T, pend_N;    /* its shape */
+    int pend_T, pend_N, pend_sums;    /* its shape */
     int pend_split;        /* how its scans were queued (which events were recorded) */
     int scan_mode;         /* OFK_SCAN_*: arithmetic of the scans of this gpubuf's decodes */
     int scan_spl;          /* states per lane of the scans, 0 = chosen from the batch size */
@@ -363,6 +363,7 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
     /* only where the search leaves the machine idle, and not with 1024 states, whose search waits for
      * memory and was measured to take half as long again beside the extra kernel */
     const int use_sums = !g->pend_split && g->path_sums != NULL && N <= OFK_SPARSE_SEARCH_MAX_CHUNKS;
+    g->pend_sums = use_sums;
     if (!g->pend_split) {
         /* both sweeps and the posterior in one kernel, then the beam search, all on one stream */
         launch_ok(ofk_scan_posterior(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, cols, stay, g->scan_mode,
@@ -378,6 +379,7 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
          * every state, so that the sequence stage reads one value per time step instead of nine. */
         if (use_sums) {
             HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BWD_END], 0));
+            HIP_OK(hipEventRecord(g->ev[EV_SUMS_START], g->s_side));
             launch_ok(ofk_path_sums(g->pub.post_NTC, g->path_sums, T, N, state_len, g->s_side), "path_sums");
             HIP_OK(hipEventRecord(g->ev[EV_SUMS_END], g->s_side));
         }
@@ -482,6 +484,8 @@ int openfish_amd_last_timings(const openfish_gpubuf_t *gpubuf, float *ms, int n)
     HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_BEAM], g->ev[EV_BEAM_START], g->ev[EV_BEAM_END]));
     HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_SEQ], g->ev[EV_SEQ_START], g->ev[EV_SEQ_END]));
     HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_TOTAL], g->ev[EV_START], g->ev[EV_SEQ_END]));
+    g->ms[OPENFISH_AMD_STAGE_SUMS] = 0.0f;
+    if (g->pend_sums) HIP_OK(hipEventElapsedTime(&g->ms[OPENFISH_AMD_STAGE_SUMS], g->ev[EV_SUMS_START], g->ev[EV_SUMS_END]));
     if (n > OPENFISH_AMD_STAGE_COUNT) n = OPENFISH_AMD_STAGE_COUNT;
     memcpy(ms, g->ms, sizeof(float) * (size_t)n);
     return n;
@@ -586,9 +590,15 @@ void openfish_amd_decode_from_tensors(int T, int N, int C, const void *scores, i
                               g->pub.moves, T, N, state_len, columns_of(C, state_len), log_beam_cut(options),
                               options->blank_score,
                               g->lse_table, g->debug_flags, g->s_main), "beam_search");
+    /* the quality stage as a whole decode runs it: from per-state sums where the gpubuf holds room for them */
+    const float *sums = NULL;
+    if (g->path_sums != NULL && N <= OFK_SPARSE_SEARCH_MAX_CHUNKS) {
+        launch_ok(ofk_path_sums(post, g->path_sums, T, N, state_len, g->s_main), "path_sums");
+        sums = g->path_sums;
+    }
     launch_ok(ofk_sequence(post, (int32_t *)g->pub.states, g->pub.moves, g->pub.qual_data, g->pub.base_probs,
                            g->pub.total_probs, g->pub.sequence, g->pub.qstring, T, N, state_len,
-                           phred_for(g, options), NULL, g->s_main), "sequence");
+                           phred_for(g, options), sums, g->s_main), "sequence");
     fetch_outputs(g, T, N, moves, sequence, qstring);
 }
 

@@ -30,7 +30,7 @@ SQ_COUNTERS = ["SQ_WAVES", "SQ_BUSY_CYCLES", "SQ_INSTS_VALU", "SQ_INSTS_SALU", "
 SCAN_MODES = {"0": "two_tier", "1": "precise", "2": "fast"}
 # kernel function -> the stage name bench.py uses
 STAGE_OF = {"scan_post_kernel": "scan", "bwd_scan_kernel": "bwd", "fwd_post_kernel": "fwd_post",
-            "beam_kernel": "beam", "sequence_kernel": "sequence"}
+            "beam_kernel": "beam", "sequence_kernel": "sequence", "path_sums_kernel": "path_sums"}
 
 
 def template_ints(name):
@@ -44,7 +44,7 @@ def template_ints(name):
 
 def short(name):
     for fn in ("scan_post_kernel", "bwd_scan_kernel", "fwd_post_kernel", "beam_kernel", "sequence_kernel",
-               "copy_kernel", "rotary_vec8_kernel", "rotary_kernel"):
+               "path_sums_kernel", "copy_kernel", "rotary_vec8_kernel", "rotary_kernel"):
         if fn in name:
             a = template_ints(name)
             if fn in ("scan_post_kernel", "bwd_scan_kernel", "fwd_post_kernel") and len(a) >= 4:

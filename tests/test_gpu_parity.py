@@ -119,6 +119,28 @@ def test_beam_stage_bit_exact_on_reference_tensors(api, name):
 
 
 @pytest.mark.parametrize("name", GPU_CASES)
+def test_quality_from_per_state_sums_equals_quality_from_gathers(api, name):
+    """the quality stage reads the posteriors behind a block either by itself (nine gathers per time
+    step: the stage-level entry point, and a decode with split scans) or as one value per time step
+    from the per-state sums a kernel leaves beside the beam search (a whole decode of up to 512
+    chunks of 64 or 256 states, and the decode from given tensors): the same fp32 sums in the same
+    order, so every output of the stage is identical bit for bit"""
+    z, sl, opt = load(name)
+    T, N, C = z["scores"].shape
+    (mv, sq, qs), gb = gpu_from_tensors(api, z["scores"], sl, opt, z["bwd"], z["post"])
+    with_sums = {k: gb.tensor(k) for k in ("qual_data", "base_probs", "total_probs", "sequence", "qstring")}
+    gb2 = api.GpuBuf(T, N, sl)
+    sc = api.upload_scores_to_hip(z["scores"])
+    rb, rp = api.DeviceBuffer.from_host(z["bwd"]), api.DeviceBuffer.from_host(z["post"])
+    o = api.DECODER_INIT(**opt)
+    api.openfish_amd_beam_search(T, N, C, sc, sl, o, rb, gb2)
+    api.openfish_amd_sequence(T, N, sl, o, rp, gb2)
+    for k, v in with_sums.items():
+        assert np.array_equal(v.view(np.uint8), gb2.tensor(k).view(np.uint8)), k
+    assert np.array_equal(sq, gb2.tensor("sequence")) and np.array_equal(qs, gb2.tensor("qstring"))
+
+
+@pytest.mark.parametrize("name", GPU_CASES)
 def test_whole_decode_on_golden(api, name):
     """openfish_decode_gpu end to end; with the CPU-faithful scan arithmetic the GPU's own
     tensors lead to the same calls as the reference's"""
