@@ -188,8 +188,12 @@ def main():
                     help="scores per state and time step: 4 (what the reference consumes) or 5 (a blank column first, "
                          "C = 5 * 4^state_len as the network emits it)")
     ap.add_argument("--scan-mode", default="two_tier", choices=("two_tier", "precise", "fast"))
-    ap.add_argument("--split-scans", action="store_true",
-                    help="backward scan, then forward scan beside the beam search, instead of both scans as one kernel")
+    ap.add_argument("--scans", default="auto", choices=("auto", "one", "split"),
+                    help="arrangement of the scans: both as one kernel, or the backward scan and then the forward scan "
+                         "beside the beam search; auto (the default): the library chooses per call")
+    ap.add_argument("--split-scans", action="store_const", dest="scans", const="split", help="the same as --scans split")
+    ap.add_argument("--states-per-lane", type=int, default=0, choices=(0, 1, 2, 4),
+                    help="force the scans' states per lane (0: the library chooses)")
     ap.add_argument("--cpu-sample", type=int, default=512, help="chunks timed on the CPU path (0 = skip; capped at N)")
     ap.add_argument("--seed", type=int, default=20251125)
     ap.add_argument("--alt-steps", type=int, default=3,
@@ -236,7 +240,9 @@ def main():
     del made, device_input
     gpubuf = api.GpuBuf(T, N, state_len)
     gpubuf.set_scan_mode(a.scan_mode)
-    gpubuf.set_split_scans(a.split_scans)
+    asked = {"auto": None, "one": False, "split": True}[a.scans]
+    gpubuf.set_split_scans(asked)
+    gpubuf.set_scan_states_per_lane(a.states_per_lane)
     call = (T, N, C, scores, state_len, opt)
 
     if a.calibrate_copy:
@@ -272,7 +278,7 @@ def main():
         gpubuf.set_scan_mode(mode)
         api.openfish_decode_gpu_discard(*call, gpubuf)
         ms, mn = timed_decodes(api, gpubuf, call, a.alt_steps)
-        gpubuf.set_split_scans(a.split_scans)
+        gpubuf.set_split_scans(asked)
         gpubuf.set_scan_mode(a.scan_mode)
         return {"chunks_per_s": round(N / (ms / 1e3), 1), "ms_per_step": round(ms, 4),
                 "stage_ms": {k: round(v, 4) for k, v in mn.items() if v > 0},
@@ -280,11 +286,12 @@ def main():
 
     other_split, fast_mode = None, None
     if a.alt_steps > 0:
-        other_split = side(not a.split_scans, a.scan_mode,
+        ran_split = mean["scan"] == 0  # what the timed calls ran with, asked for or chosen by the library
+        other_split = side(not ran_split, a.scan_mode,
                            "split scans: backward scan, then forward scan + posterior on a second stream beside the beam search"
-                           if not a.split_scans else "both scans and the posterior as one kernel, then the beam search")
+                           if not ran_split else "both scans and the posterior as one kernel, then the beam search")
         if a.scan_mode != "fast":
-            fast_mode = side(a.split_scans, "fast",
+            fast_mode = side(asked, "fast",
                              "scans with v_exp_f32/v_log_f32 only: bwd within 2 ulp, a few posteriors per ten million "
                              "beyond 1e-3 relative; outside the acceptance bar, shown as the memory-bound floor of the kernels")
 
@@ -309,7 +316,7 @@ def main():
     if a.overlap_steps > 0:
         bufs = [gpubuf, api.GpuBuf(T, N, state_len)]
         bufs[1].set_scan_mode(a.scan_mode)
-        bufs[1].set_split_scans(a.split_scans)
+        bufs[1].set_split_scans(asked)
         api.openfish_decode_gpu(*call, bufs[1])
         t2 = time.perf_counter()
         api.openfish_amd_decode_enqueue(*call, bufs[0])

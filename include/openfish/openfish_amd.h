@@ -204,11 +204,12 @@ int openfish_amd_last_timings(const openfish_gpubuf_t *gpubuf, float *ms, int n)
  *   (state & 15) instead of the state, so that different sequences share hashes and that route
  *   is found by the search's own duplicate detection; for tests against a CPU search seeded
  *   the same way, never for real decoding.
- * split scans: 0 (default) runs both scans and the posterior as one kernel, then the beam
- *   search; 1 runs the backward scan, then the forward scan + posterior on a second stream
- *   beside the beam search.  Same results.  The first arrangement has the shorter scan stage at
- *   every batch size; the second one hides the forward scan beneath the beam search and can
- *   come out ahead for blocking calls on small batches.
+ * split scans: 0 runs both scans and the posterior as one kernel, then the beam search; 1 runs the
+ *   backward scan, then the forward scan + posterior on a second stream beside the beam search.
+ *   Same results.  The first arrangement has the shorter scan stage at every batch size; the second
+ *   hides the forward scan beneath the beam search, which pays while that search, one wavefront per
+ *   chunk, leaves the machine idle.  A negative value, the default, lets every call choose: split
+ *   for up to 512 chunks of 256 states (2048 of 64), one kernel beyond that and for 1024 states.
  */
 void openfish_amd_gpubuf_set_scan_mode(const openfish_gpubuf_t *gpubuf, int scan_mode);
 void openfish_amd_gpubuf_set_split_scans(const openfish_gpubuf_t *gpubuf, int split);

@@ -204,7 +204,9 @@ class GpuBuf:
         _L.openfish_amd_gpubuf_set_scan_mode(self.handle, SCAN_MODES.get(mode, mode))
 
     def set_split_scans(self, split):
-        _L.openfish_amd_gpubuf_set_split_scans(self.handle, 1 if split else 0)
+        """True: backward scan, then forward scan + posterior beside the beam search; False: both
+        scans as one kernel; None: the library chooses per call (the default)"""
+        _L.openfish_amd_gpubuf_set_split_scans(self.handle, -1 if split is None else (1 if split else 0))
 
     def set_scan_states_per_lane(self, spl):
         _L.openfish_amd_gpubuf_set_scan_states_per_lane(self.handle, int(spl))

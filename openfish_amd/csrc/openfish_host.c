@@ -138,7 +138,8 @@ typedef struct {
     int scan_mode;         /* OFK_SCAN_*: arithmetic of the scans of this gpubuf's decodes */
     int scan_spl;          /* states per lane of the scans, 0 = chosen from the batch size */
     int debug_flags;       /* bit 0: serial replay of the beam search's merges; bit 1: colliding seed hashes */
-    int split_scans;       /* 1: backward sweep, then forward sweep beside the beam search; 0: both sweeps in one kernel */
+    int split_scans;       /* 1: backward sweep, then forward sweep beside the beam search; 0: both sweeps in one
+                            * kernel; -1 (default): chosen per call by split_by_default() */
     ofk_phred_table_t phred; /* thresholds for (phred_shift, phred_scale) */
     float phred_shift, phred_scale;
     int phred_valid;
@@ -164,6 +165,7 @@ openfish_gpubuf_t *openfish_gpubuf_init(const int T, const int N, const int stat
     g->T = T;
     g->N = N;
     g->state_len = state_len;
+    g->split_scans = -1;
 
     /* field sizes as in the reference (src/decode_hip.hip:24-48) except beam_vector,
      * whose slots are 2 bytes here */
@@ -349,6 +351,19 @@ static void join_null_stream(ofa_gpubuf_t *g) {
     HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_JOIN], 0));
 }
 
+/* Which arrangement of the scans a blocking decode finishes sooner with, as measured on whole
+ * decodes (T = 1666; chunks/s with one kernel | split):
+ *     64 states:  512 chunks 248k | 260k, 2048 chunks 418k | 485k
+ *    256 states:  128 chunks  57k |  61k,  512 chunks 180k | 195k, 1024 chunks 215k | 206k, 2048 chunks 223k | 207k
+ *   1024 states:   64 chunks 16.6k | 16.9k, 256 chunks 57.7k | 55.2k
+ * Up to 512 chunks of 256 states (or as many states in all with 64 per chunk) the beam search, one
+ * wave per chunk, is the longest stage and leaves most of the machine idle: the forward sweep and the
+ * posterior fit beside it.  Beyond that the search fills the compute units itself and the one
+ * kernel, which has the shorter scan stage at every size, wins. */
+static int split_by_default(int N, int state_len) {
+    return state_len <= 4 && (long)N * states_of(state_len) <= 512L * 256L;
+}
+
 /* Queue one decode on the gpubuf's streams, results into its pinned staging buffer; returns
  * without waiting for the GPU. */
 static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int C, const void *scores_TNC,
@@ -359,7 +374,7 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
     join_null_stream(g);
     HIP_OK(hipEventRecord(g->ev[EV_START], g->s_main));
     const int cols = columns_of(C, state_len);
-    g->pend_split = g->split_scans;
+    g->pend_split = g->split_scans < 0 ? split_by_default(N, state_len) : g->split_scans;
     /* only where the search leaves the machine idle, and not with 1024 states, whose search waits for
      * memory and was measured to take half as long again beside the extra kernel */
     const int use_sums = !g->pend_split && g->path_sums != NULL && N <= OFK_SPARSE_SEARCH_MAX_CHUNKS;
@@ -722,7 +737,7 @@ void openfish_amd_gpubuf_set_scan_mode(const openfish_gpubuf_t *gpubuf, int scan
 }
 
 void openfish_amd_gpubuf_set_split_scans(const openfish_gpubuf_t *gpubuf, int split) {
-    owned(gpubuf)->split_scans = split ? 1 : 0;
+    owned(gpubuf)->split_scans = split < 0 ? -1 : (split ? 1 : 0);
 }
 
 void openfish_amd_gpubuf_set_scan_states_per_lane(const openfish_gpubuf_t *gpubuf, int spl) {

@@ -1031,13 +1031,14 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 // that still gives every SIMD of the device (256 CUs x 4) a wave; small batches are
 // spread thinner.  1024 states at one state per lane would need 1024-thread groups
 // with a barrier per step, so that size stops at 2.
-// The backward sweep of the smaller models measures faster with two waves per SIMD
-// (hac, 512 chunks: 1.29 ms against 1.33 ms; 0.56 against 0.68 ms with hardware exp/log).
+// The sweeps of the smaller models measure faster with two waves per SIMD (hac, 512 chunks:
+// backward 1.29 ms against 1.33 ms; forward + posterior beside the beam search 1.41 ms against
+// 1.61 ms, which is 13 000 chunks/s of a whole decode).
 // `forced` = 4, 2 or 1 overrides the choice (0 = choose).
 int states_per_lane(int S, int N, bool backward, int forced) {
     const int min_spl = S >= 1024 ? 2 : 1;
     if (forced == 4 || forced == 2 || forced == 1) return forced < min_spl ? min_spl : forced;
-    const long wanted = (backward && S <= 256) ? 2048 : 1024;
+    const long wanted = S <= 256 ? 2048 : 1024;
     for (int spl = 4; spl > min_spl; spl >>= 1) {
         const long waves = ((long)N * (S / spl) + 63) / 64;
         if (waves >= wanted) return spl;

@@ -140,7 +140,9 @@ def main():
             except (OSError, ValueError):
                 whole = {}
             table["bench_args"] = args
-            whole[a.traffic_key] = table
+            merged = whole.get(a.traffic_key, {})  # runs of both scan arrangements fill one entry
+            merged.update(table)
+            whole[a.traffic_key] = merged
             with open(a.traffic_json, "w") as fh:
                 json.dump(whole, fh, indent=1, sort_keys=True)
                 fh.write("\n")

@@ -151,11 +151,21 @@ def test_whole_decode_on_golden(api, name):
         pytest.skip("the CPU scans ignore blank_score, the GPU entry point does not (as in the reference)")
     sc = api.upload_scores_to_hip(s16)
     gb = api.GpuBuf(T, N, sl)
-    mv, sq, qs = api.openfish_decode_gpu(T, N, C, sc, sl, api.DECODER_INIT(**opt), gb)
-    assert np.array_equal(mv, z["moves"]) and np.array_equal(sq, z["sequence"]) and np.array_equal(qs, z["qstring"])
-    t = gb.timings()
-    assert set(t) == set(api.STAGES) and t["beam"] > 0 and t["sequence"] > 0 and t["total"] > 0
-    assert t["scan"] > 0 and t["bwd"] == 0 and t["fwd_post"] == 0  # both scans ran as one kernel
+    for split in (None, False, True):  # the library's choice for the batch, one kernel, two kernels
+        gb.set_split_scans(split)
+        mv, sq, qs = api.openfish_decode_gpu(T, N, C, sc, sl, api.DECODER_INIT(**opt), gb)
+        assert np.array_equal(mv, z["moves"]) and np.array_equal(sq, z["sequence"]) and np.array_equal(qs, z["qstring"])
+        t = gb.timings()
+        assert set(t) == set(api.STAGES) and t["beam"] > 0 and t["sequence"] > 0 and t["total"] > 0
+        ran_split = t["scan"] == 0
+        if ran_split:
+            assert t["bwd"] > 0 and t["fwd_post"] > 0 and t["path_sums"] == 0
+        else:
+            assert t["bwd"] == 0 and t["fwd_post"] == 0 and (t["path_sums"] > 0) == (sl <= 4 and N <= 512)
+        if split is None:  # small batches of up to 256 states run split
+            assert ran_split == (sl <= 4 and N * 4 ** sl <= 512 * 256)
+        else:
+            assert ran_split == split
 
 
 def test_reference_in_repo_fixture_end_to_end(api):
