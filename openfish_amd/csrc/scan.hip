@@ -575,6 +575,142 @@ __global__ __launch_bounds__((Shape<S, SPL>::kThreads)) void fwd_post_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// forward + posterior with the two jobs on different waves.
+//
+// fwd_post_kernel's lanes take the posterior of a row between two steps of the recursion: an
+// exponential, a sum over the wave, a partial sum through LDS, a reciprocal and a store join the
+// chain of dependent operations of every time step, which is what this sweep's duration is made
+// of (it runs beside the beam search with two waves per SIMD; 512 chunks of 256 states: 1.41 ms
+// against 0.95 ms for the backward sweep, which has no such work).  Here a chunk has twice the
+// lanes: one half runs the recursion alone, the other half reads every row the first half
+// publishes in LDS for its own exchange anyway, and forms that row's posterior one step behind.
+// Every wave takes one block barrier per time step (plus one at the end and two for the shift).
+// Same arithmetic, same results.  (Letting the second half also sum the finished row over every
+// state's neighbours for the quality stage was measured and dropped: the extra LDS traffic slowed
+// the recursion by more, 0.18 ms, than the sums save that stage, 0.09 ms.)
+// ---------------------------------------------------------------------------
+template <int S, int SPL, int DEPTH>
+__global__ __launch_bounds__((2 * (S / SPL))) void fwd_post_roles_kernel(
+    const _Float16 *__restrict__ scores, const float *__restrict__ bwd, float *__restrict__ post, int T,
+    int N, float stay, LogSeries series) {
+    constexpr int L = S / SPL;  // lanes of either job
+    constexpr int Q = S / 4;
+    constexpr int RW = L / 64;  // waves of either job
+    static_assert(L % 64 == 0 && RW > 1, "either job owns several whole waves");
+    __shared__ __attribute__((aligned(16))) float vec[2][S];
+    __shared__ float part[2][RW];
+    __shared__ __attribute__((aligned(16))) ofa::LogCell logcells[32];
+    __shared__ __attribute__((aligned(16))) float tier_lanes[L];
+    const int tid = threadIdx.x;
+    const int posterior = __builtin_amdgcn_readfirstlane(tid / L);
+    const int l = tid % L, lane = tid & 63, wave = l / 64;
+    const LogArgs logtab{logcells, series.c, series.e, tier_lanes + (l & ~63)};
+    if (tid < 32) logcells[tid] = ofa::log_cell(tid);
+    const int s0 = SPL * l, q = s0 >> 2;  // own states s0 .. s0+SPL-1, all in quad q
+    const int n = blockIdx.x;            // one chunk per workgroup
+    const size_t row_stride = (size_t)N * kCols * S;
+    auto barrier = [] { chunk_sync<true>(); };
+
+    if (!posterior) {
+        const _Float16 *sp = scores + (size_t)n * kCols * S + kCols * s0 + kLead;
+        FwdRow<SPL> ring[DEPTH];
+#pragma unroll
+        for (int k = 0; k < DEPTH; ++k) {
+            if (k < T) ring[k].load(sp + (size_t)k * row_stride);
+        }
+        float f[SPL];
+#pragma unroll
+        for (int i = 0; i < SPL; ++i) f[i] = 0.f;
+        int buf = 0;
+        barrier();  // the other half exchanges the maxima behind the shift
+        barrier();
+        __syncthreads();  // the log table
+        for (int done = 0; done <= T; done += DEPTH) {
+#pragma unroll
+            for (int k = 0; k < DEPTH; ++k) {
+                const int t = done + k;
+                if (t <= T) {
+                    const FwdRow<SPL> row = ring[k];
+                    if (t + DEPTH < T) ring[k].load(sp + (size_t)(t + DEPTH) * row_stride);
+                    FloatRun<SPL> mine;
+#pragma unroll
+                    for (int i = 0; i < SPL; ++i) mine.v[i] = f[i];
+                    mine.store(&vec[buf][s0]);  // row t
+                    barrier();
+                    if (t < T) {
+                        const float p0 = vec[buf][q], p1 = vec[buf][q + Q];
+                        const float p2 = vec[buf][q + 2 * Q], p3 = vec[buf][q + 3 * Q];
+                        fwd_update<0, SPL, OFK_SCAN_TWO_TIER>(f, p0, p1, p2, p3, row, stay, logtab);
+                        buf ^= 1;
+                    }
+                }
+            }
+        }
+        barrier();  // the other half finishes row T
+    } else {
+        const float *bp = bwd + (size_t)n * (size_t)(T + 1) * S + s0;
+        float *pp = post + (size_t)n * (size_t)(T + 1) * S + s0;
+        FloatRun<SPL> bring[DEPTH];
+#pragma unroll
+        for (int k = 0; k < DEPTH; ++k) {
+            if (k <= T) bring[k].load(bp + (size_t)k * S);
+        }
+        // Shift of the softmax exponent, as in fwd_post_kernel: max_s bwd[0][s] - 10.
+        float shift;
+        {
+            float m = bring[0].v[0];
+#pragma unroll
+            for (int i = 1; i < SPL; ++i) m = fmaxf(m, bring[0].v[i]);
+            m = group_max<64>(m);
+            if (lane == 0) part[0][wave] = m;
+            barrier();
+            m = part[0][0];
+#pragma unroll
+            for (int w = 1; w < RW; ++w) m = fmaxf(m, part[0][w]);
+            barrier();
+            shift = m - 10.0f;
+        }
+        __syncthreads();
+        FloatRun<SPL> e;  // terms of the row before, waiting for the sum over the waves
+        int buf = 0;
+        auto finish_row = [&](int t) {
+            float total = part[t & 1][0];
+#pragma unroll
+            for (int w = 1; w < RW; ++w) total += part[t & 1][w];
+            const float inv = __builtin_amdgcn_rcpf(total);
+#pragma unroll
+            for (int i = 0; i < SPL; ++i) e.v[i] *= inv;
+            e.store(pp + (size_t)t * S);
+        };
+        for (int done = 0; done <= T; done += DEPTH) {
+#pragma unroll
+            for (int k = 0; k < DEPTH; ++k) {
+                const int t = done + k;
+                if (t <= T) {
+                    const FloatRun<SPL> bw = bring[k];
+                    if (t + DEPTH <= T) bring[k].load(bp + (size_t)(t + DEPTH) * S);
+                    barrier();  // row t is in vec[buf], the partial sums of row t - 1 in part[(t - 1) & 1]
+                    if (t > 0) finish_row(t - 1);
+                    FloatRun<SPL> fv;
+                    fv.load(&vec[buf][s0]);
+                    buf ^= 1;
+                    float total = 0.f;
+#pragma unroll
+                    for (int i = 0; i < SPL; ++i) {
+                        e.v[i] = __builtin_amdgcn_exp2f(((fv.v[i] + bw.v[i]) - shift) * kLog2e);
+                        total += e.v[i];
+                    }
+                    total = group_sum<64>(total);
+                    if (lane == 0) part[t & 1][wave] = total;
+                }
+            }
+        }
+        barrier();
+        finish_row(T);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Both sweeps in one kernel, meeting in the middle.
 //
 // The forward recursion does not depend on the backward one; only the posterior needs
@@ -980,6 +1116,16 @@ int launch_fwd(int mode, const void *scores, const float *bwd, float *post, int 
     const _Float16 *sc = static_cast<const _Float16 *>(scores);
     switch (mode) {
         case OFK_SCAN_TWO_TIER:
+            // Recursion and posterior on separate waves, one chunk per group of twice the lanes: where a chunk
+            // spans several waves, and while that leaves every SIMD at most four of them (measured, 256 states:
+            // 512 chunks 1.17 ms against 1.41 ms beside the beam search, 1024 chunks 3.5 against 3.1)
+            if constexpr (Sh::kMultiWave && 2 * Sh::kLanes <= 1024) {
+                if ((long)N * (2 * Sh::kLanes / 64) <= 4096) {
+                    hipLaunchKernelGGL((fwd_post_roles_kernel<S, SPL, DEPTH>), dim3(N), dim3(2 * Sh::kLanes), 0, st, sc, bwd, post,
+                                       T, N, stay, kSeries);
+                    break;
+                }
+            }
             hipLaunchKernelGGL((fwd_post_kernel<S, SPL, DEPTH, OFK_SCAN_TWO_TIER>), grid, block, 0, st, sc, bwd, post, T, N, stay, kSeries);
             break;
         case OFK_SCAN_PRECISE:

@@ -29,7 +29,7 @@ SQ_COUNTERS = ["SQ_WAVES", "SQ_BUSY_CYCLES", "SQ_INSTS_VALU", "SQ_INSTS_SALU", "
                "SQ_LDS_BANK_CONFLICT", "SQ_ACTIVE_INST_VALU"]
 SCAN_MODES = {"0": "two_tier", "1": "precise", "2": "fast"}
 # kernel function -> the stage name bench.py uses
-STAGE_OF = {"scan_post_kernel": "scan", "bwd_scan_kernel": "bwd", "fwd_post_kernel": "fwd_post",
+STAGE_OF = {"scan_post_kernel": "scan", "bwd_scan_kernel": "bwd", "fwd_post_kernel": "fwd_post", "fwd_post_roles_kernel": "fwd_post",
             "beam_kernel": "beam", "sequence_kernel": "sequence", "path_sums_kernel": "path_sums"}
 
 
@@ -43,10 +43,12 @@ def template_ints(name):
 
 
 def short(name):
-    for fn in ("scan_post_kernel", "bwd_scan_kernel", "fwd_post_kernel", "beam_kernel", "sequence_kernel",
-               "path_sums_kernel", "copy_kernel", "rotary_vec8_kernel", "rotary_kernel"):
+    for fn in ("scan_post_kernel", "bwd_scan_kernel", "fwd_post_roles_kernel", "fwd_post_kernel", "beam_kernel",
+               "sequence_kernel", "path_sums_kernel", "copy_kernel", "rotary_vec8_kernel", "rotary_kernel"):
         if fn in name:
             a = template_ints(name)
+            if fn == "fwd_post_roles_kernel" and len(a) >= 3:
+                return "%s<S=%s,SPL=%s,DEPTH=%s>" % (fn, a[0], a[1], a[2])
             if fn in ("scan_post_kernel", "bwd_scan_kernel", "fwd_post_kernel") and len(a) >= 4:
                 return "%s<S=%s,SPL=%s,DEPTH=%s,%s>" % (fn, a[0], a[1], a[2], SCAN_MODES.get(a[3], a[3]))
             if fn == "beam_kernel" and len(a) >= 3:
