@@ -11,6 +11,8 @@ OUT_DIR holds one sub-directory per pass, each written by one rocprofv3 run of t
     write/   rocprofv3 --pmc WRITE_SIZE       --output-format csv -d OUT_DIR/write -o w -- python3 bench.py ...
     sq/      rocprofv3 --pmc SQ_WAVES SQ_BUSY_CYCLES SQ_INSTS_VALU SQ_INSTS_SALU SQ_INSTS_LDS SQ_WAIT_INST_LDS
                        SQ_LDS_BANK_CONFLICT SQ_ACTIVE_INST_VALU --output-format csv -d OUT_DIR/sq -o s -- ...
+    sq2/     rocprofv3 --pmc SQ_WAVE_CYCLES SQ_WAIT_ANY SQ_ACTIVE_INST_ANY SQ_ACTIVE_INST_LDS SQ_INSTS_VALU_FMA_F64
+                       SQ_INSTS_VALU_TRANS_F32 SQ_INSTS_BRANCH SQ_WAIT_INST_ANY --output-format csv -d OUT_DIR/sq2 -o s -- ...
 
 FETCH_SIZE and WRITE_SIZE are scaled by what the same counters read for the library's plain copy
 kernel, which bench.py launches once when given --calibrate-copy MIB (MIB read, MIB written).
@@ -27,6 +29,8 @@ import re
 
 SQ_COUNTERS = ["SQ_WAVES", "SQ_BUSY_CYCLES", "SQ_INSTS_VALU", "SQ_INSTS_SALU", "SQ_INSTS_LDS", "SQ_WAIT_INST_LDS",
                "SQ_LDS_BANK_CONFLICT", "SQ_ACTIVE_INST_VALU"]
+SQ2_COUNTERS = ["SQ_WAVE_CYCLES", "SQ_WAIT_ANY", "SQ_ACTIVE_INST_ANY", "SQ_ACTIVE_INST_LDS", "SQ_INSTS_VALU_FMA_F64",
+                "SQ_INSTS_VALU_TRANS_F32", "SQ_INSTS_BRANCH", "SQ_WAIT_INST_ANY"]
 SCAN_MODES = {"0": "two_tier", "1": "precise", "2": "fast"}
 # kernel function -> the stage name bench.py uses
 STAGE_OF = {"scan_post_kernel": "scan", "bwd_scan_kernel": "bwd", "fwd_post_kernel": "fwd_post", "fwd_post_roles_kernel": "fwd_post",
@@ -86,6 +90,8 @@ def main():
                                                            "profiles", "traffic.json"))
     ap.add_argument("--updates", type=float, default=0,
                     help="state updates of one scan sweep per launch (N * T * S): adds VALU instructions per update")
+    ap.add_argument("--steps-per-wave", type=float, default=0,
+                    help="time steps T every scan wave takes: adds fp64 FMA per wave and time step")
     a = ap.parse_args()
 
     base, args = a.out_dir, a.bench_args
@@ -96,6 +102,7 @@ def main():
            "rocprofv3 --pmc FETCH_SIZE --output-format csv -d OUT/fetch -o f -- python3 bench.py A",
            "rocprofv3 --pmc WRITE_SIZE --output-format csv -d OUT/write -o w -- python3 bench.py A",
            "rocprofv3 --pmc %s --output-format csv -d OUT/sq -o s -- python3 bench.py A" % " ".join(SQ_COUNTERS),
+           "rocprofv3 --pmc %s --output-format csv -d OUT/sq2 -o s -- python3 bench.py A" % " ".join(SQ2_COUNTERS),
            "python3 -m openfish_amd.profile_report OUT --title ... --bench-args \"A\" --md <this file>",
            "```\n"]
 
@@ -167,6 +174,35 @@ def main():
             out.append("\nVALU per state update = SQ_INSTS_VALU (wave instructions) x 64 lanes / (sweeps x N x T x S state "
                        "updates): the vector instructions one lane issues for one update of one state, everything "
                        "around the update (loads, posterior, exchange through LDS) included.")
+
+    sq2 = first(os.path.join(base, "sq2", "**", "*counter_collection.csv"))
+    if sq and sq2:
+        c1, c2 = counters(sq), counters(sq2)
+        out.append("\n## Where the waves' time goes (`--pmc %s`, with the table above)\n" % " ".join(SQ2_COUNTERS))
+        out.append("Per launch. The SQ's time counters tick once per four clocks; WAVE_CYCLES adds up the lifetimes of all "
+                   "waves, ACTIVE_INST_VALU the time their vector instructions occupy a SIMD's ALU. `VALU share of wave "
+                   "time` x `waves per SIMD` is the fraction of time a SIMD's vector ALU is busy (1024 SIMDs; the waves of "
+                   "these kernels are all resident at once).\n")
+        out.append("| kernel | WAVE_CYCLES | WAIT_ANY | ACTIVE_INST_ANY | ACTIVE_INST_LDS | INSTS_VALU_FMA_F64 | INSTS_VALU_TRANS_F32 | "
+                   "INSTS_BRANCH | VALU share of wave time | waves per SIMD | SIMD vector ALU busy | fp64 FMA per wave and time step |"
+                   "\n|---|---|---|---|---|---|---|---|---|---|---|---|")
+        for k, d in c2.items():
+            if k.startswith("__amd") or k not in c1:
+                continue
+            wc, act, waves = d.get("SQ_WAVE_CYCLES", 0.0), c1[k].get("SQ_ACTIVE_INST_VALU", 0.0), c1[k].get("SQ_WAVES", 0.0)
+            share = act / wc if wc else 0.0
+            per_simd = waves / 1024.0
+            steps = a.steps_per_wave
+            out.append("| %s | %.3g | %.3g | %.3g | %.3g | %.3g | %.3g | %.3g | %.3f | %.2f | %.2f | %s |" % (
+                k, wc, d.get("SQ_WAIT_ANY", 0.0), d.get("SQ_ACTIVE_INST_ANY", 0.0), d.get("SQ_ACTIVE_INST_LDS", 0.0),
+                d.get("SQ_INSTS_VALU_FMA_F64", 0.0), d.get("SQ_INSTS_VALU_TRANS_F32", 0.0), d.get("SQ_INSTS_BRANCH", 0.0),
+                share, per_simd, min(1.0, share * per_simd),
+                ("%.2f" % (d.get("SQ_INSTS_VALU_FMA_F64", 0.0) / (waves * steps))) if (steps and waves and stage_of(k) in ("scan", "bwd", "fwd_post")) else "-"))
+        if a.steps_per_wave:
+            out.append("\nfp64 FMA per wave and time step = SQ_INSTS_VALU_FMA_F64 / (waves x T): the second tier of the default "
+                       "arithmetic is the only user of fp64 in the scans besides the 32 warm-up steps of either sweep (70 fp64 "
+                       "FMA per wave and step there); one trip through it is 23 fp64 FMA, so the figure, less the warm-up's "
+                       "share, over 23 is the number of trips per wave-level update.")
 
     log = first(os.path.join(base, "trace.log"))
     if log:
