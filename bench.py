@@ -264,6 +264,15 @@ def main():
             stages[k] = {"ms": round(mean[k], 4), "algorithmic_GB": round(need[k] / 1e9, 4),
                          "GBps": round(need[k] / 1e9 / (mean[k] / 1e3), 1)}
     stages["device_total_ms"] = round(mean["total"], 4)
+    # kernels that share the machine: the beam search starts together with the forward scan (split scans) or
+    # with the path sums (one scan kernel); their algorithmic bytes over the longer of the two
+    beside = "fwd_post" if mean["fwd_post"] > 0 else ("path_sums" if mean["path_sums"] > 0 else None)
+    if beside:
+        window_ms = max(mean["beam"], mean[beside])
+        gb = (need["beam"] + need[beside]) / 1e9
+        stages["beam_and_" + beside + "_side_by_side"] = {
+            "ms": round(window_ms, 4), "algorithmic_GB": round(gb, 4), "GBps": round(gb / (window_ms / 1e3), 1),
+            "frac_of_hbm_peak": round(gb / (window_ms / 1e3) / HBM_PEAK_GBS, 4)}
     stages["scan_plus_posterior"] = scan_stage(need, mean)
     scan_gbs = stages["scan_plus_posterior"]["GBps"]
     dominant = max((k for k in ("scan", "bwd", "fwd_post", "beam", "sequence") if k in stages), key=lambda k: stages[k]["ms"])

@@ -11,6 +11,11 @@
  * 1666 unless given.  Writes moves.blob, sequence.blob and qstring.blob (N*T bytes
  * each) into the current directory; with OPENFISH_DUMP_TENSORS=1 also the device
  * tensors (bwd_NTC, post_NTC, qual_data, base_probs, total_probs).
+ *
+ * OPENFISH_BENCH_BATCHES=<n> decodes the batch n times and reports the time of all of them, the
+ * job of the reference driver's BENCH build (src/main.c:274-298; built with -DBENCH this driver takes
+ * the reference's counts, 1400 / 3450 / 6850 batches for state_len 3 / 4 / 5, 140 otherwise, unless
+ * the variable says otherwise).  The files hold the last batch's results.
  */
 #include <errno.h>
 #include <stdio.h>
@@ -105,13 +110,31 @@ int main(int argc, char *argv[]) {
     else if (state_len == 4) { options.q_scale = 0.95f; options.q_shift = -0.2f; }
     else { options.q_scale = 0.95f; options.q_shift = 0.5f; }
 
-    uint8_t *moves;
-    char *sequence, *qstring;
+    long n_batch = 1;
+#ifdef BENCH
+    n_batch = state_len == 3 ? 1400 : state_len == 4 ? 3450 : state_len == 5 ? 6850 : 140;
+#endif
+    const char *batches = getenv("OPENFISH_BENCH_BATCHES");
+    if (batches && atol(batches) > 0) n_batch = atol(batches);
+
+    uint8_t *moves = NULL;
+    char *sequence = NULL, *qstring = NULL;
     struct timespec t0, t1;
     clock_gettime(CLOCK_MONOTONIC, &t0);
-    openfish_decode_gpu(T, N, C, scores_gpu, state_len, &options, gpubuf, &moves, &sequence, &qstring);
+    for (long i = 0; i < n_batch; ++i) {
+        if (i) {
+            free(moves);
+            free(sequence);
+            free(qstring);
+        }
+        openfish_decode_gpu(T, N, C, scores_gpu, state_len, &options, gpubuf, &moves, &sequence, &qstring);
+    }
     clock_gettime(CLOCK_MONOTONIC, &t1);
-    OPENFISH_LOG_DEBUG("decode completed in %f secs", (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec));
+    const double secs = (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
+    OPENFISH_LOG_DEBUG("decode completed in %f secs", secs);
+    if (n_batch > 1)
+        fprintf(stderr, "openfish: %ld batches of %d chunks in %f secs (%.0f chunks/s)\n", n_batch, N, secs,
+                (double)n_batch * N / secs);
 
     const size_t nt = (size_t)N * (size_t)T;
     write_blob("moves.blob", moves, nt);

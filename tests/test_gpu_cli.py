@@ -36,6 +36,20 @@ def test_reference_fixture_through_the_cli(api, tmp_path):
         assert np.array_equal(got, want), name
 
 
+def test_cli_repeats_the_batch_like_the_reference_s_bench_build(api, tmp_path):
+    """OPENFISH_BENCH_BATCHES=n decodes the batch n times (the reference driver's BENCH loop): same
+    files as one decode, and a line with the rate"""
+    env = dict(os.environ, OPENFISH_BENCH_BATCHES="5")
+    r = subprocess.run([CLI, os.path.join(GOLDEN, "ref_fixture_scores.blob"), "1", "3"], cwd=tmp_path,
+                       capture_output=True, text=True, timeout=120, env=env)
+    assert r.returncode == 0, r.stderr
+    assert "5 batches of 1 chunks" in r.stderr
+    for name in ("moves", "sequence", "qstring"):
+        got = np.fromfile(tmp_path / (name + ".blob"), np.uint8)
+        want = np.fromfile(os.path.join(GOLDEN, "ref_fixture_%s.blob" % name), np.uint8)
+        assert np.array_equal(got, want), name
+
+
 def test_cli_converts_fp32_blobs_like_numpy_and_dumps_tensors(api, tmp_path):
     T, N, sl = 60, 3, 3
     rng = np.random.default_rng(8)
