@@ -377,7 +377,11 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
     g->pend_split = g->split_scans < 0 ? split_by_default(N, state_len) : g->split_scans;
     /* only where the search leaves the machine idle, and not with 1024 states, whose search waits for
      * memory and was measured to take half as long again beside the extra kernel */
-    const int use_sums = !g->pend_split && g->path_sums != NULL && N <= OFK_SPARSE_SEARCH_MAX_CHUNKS;
+    /* With split scans the posteriors are complete when the forward kernel ends.  With 64 states that is
+     * well before the search does (0.83 against 1.13 ms at 512 chunks), and the sums (0.21 ms) fit in
+     * between; with 256 states the two end together and the sequence stage gathers by itself. */
+    const int sums_fit = g->path_sums != NULL && N <= OFK_SPARSE_SEARCH_MAX_CHUNKS;
+    const int use_sums = sums_fit && (!g->pend_split || state_len == 3);
     g->pend_sums = use_sums;
     if (!g->pend_split) {
         /* both sweeps and the posterior in one kernel, then the beam search, all on one stream */
@@ -420,10 +424,15 @@ static void enqueue_decode(ofa_gpubuf_t *g, const int T, const int N, const int 
         launch_ok(ofk_fwd_post_scan(scores_TNC, g->pub.bwd_NTC, g->pub.post_NTC, T, N, state_len, cols, stay, g->scan_mode,
                                     g->scan_spl, g->s_side), "fwd_post_scan");
         HIP_OK(hipEventRecord(g->ev[EV_FWD_END], g->s_side));
+        if (use_sums) {
+            HIP_OK(hipEventRecord(g->ev[EV_SUMS_START], g->s_side));
+            launch_ok(ofk_path_sums(g->pub.post_NTC, g->path_sums, T, N, state_len, g->s_side), "path_sums");
+            HIP_OK(hipEventRecord(g->ev[EV_SUMS_END], g->s_side));
+        }
         /* the moves are final once the beam search is: they travel while the sequence stage runs */
         HIP_OK(hipStreamWaitEvent(g->s_side, g->ev[EV_BEAM_END], 0));
         HIP_OK(hipMemcpyAsync(g->h_out, g->pub.moves, nt, hipMemcpyDeviceToHost, g->s_side));
-        HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[EV_FWD_END], 0));
+        HIP_OK(hipStreamWaitEvent(g->s_main, g->ev[use_sums ? EV_SUMS_END : EV_FWD_END], 0));
     }
 
     HIP_OK(hipEventRecord(g->ev[EV_SEQ_START], g->s_main));

@@ -158,8 +158,8 @@ def test_whole_decode_on_golden(api, name):
         t = gb.timings()
         assert set(t) == set(api.STAGES) and t["beam"] > 0 and t["sequence"] > 0 and t["total"] > 0
         ran_split = t["scan"] == 0
-        if ran_split:
-            assert t["bwd"] > 0 and t["fwd_post"] > 0 and t["path_sums"] == 0
+        if ran_split:  # the sums follow the forward kernel where they fit beside the search: 64 states
+            assert t["bwd"] > 0 and t["fwd_post"] > 0 and (t["path_sums"] > 0) == (sl == 3 and N <= 512)
         else:
             assert t["bwd"] == 0 and t["fwd_post"] == 0 and (t["path_sums"] > 0) == (sl <= 4 and N <= 512)
         if split is None:  # small batches of up to 256 states run split
