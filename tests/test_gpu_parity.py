@@ -268,6 +268,30 @@ def test_random_shapes_whole_decode(api, seed):
         qstring_close(qs, ref["qstring"], mv)
 
 
+@pytest.mark.parametrize("state_len,T,N,five", [(4, 96, 2048, False), (4, 40, 2048, True), (3, 50, 2100, False),
+                                                 (5, 24, 512, False)])
+def test_batches_whose_rows_lie_4_mib_apart_whole_decode(api, state_len, T, N, five):
+    """short chunks in batches where one time step of the scores is 4 MiB (2048 chunks of 256 states, 512 of
+    1024; 5 MiB with five columns), the spacing at which the rows a workgroup keeps in flight share DRAM
+    banks, and beyond 2048 chunks of 64 states: in every arrangement setting the whole decode gives the
+    oracle's bwd, moves and sequence, posteriors within tolerance, phred string within qstring_close"""
+    S = 4 ** state_len
+    out = synth.crf_scores(T, N, state_len, seed=77 + N + T, chunk_scale=synth.stress_scale(N), five_columns=five,
+                           threads=16)
+    four, dev_in = (out[0], out[1]) if five else (out, out)
+    kw = dict(q_scale=0.95, q_shift=-0.2)
+    ref = O.decode(four.astype(np.float32), state_len, kw, nthreads=16)
+    gb = api.GpuBuf(T, N, state_len)
+    sc = api.upload_scores_to_hip(dev_in)
+    for split in (None, False, True):
+        gb.set_split_scans(split)
+        mv, sq, qs = api.openfish_decode_gpu(T, N, (5 if five else 4) * S, sc, state_len, api.DECODER_INIT(**kw), gb)
+        assert np.array_equal(gb.tensor("bwd_NTC"), ref["bwd"]), split
+        close(gb.tensor("post_NTC"), ref["post"], POST_ATOL)
+        assert np.array_equal(mv, ref["moves"]) and np.array_equal(sq, ref["sequence"]), split
+        qstring_close(qs, ref["qstring"], mv)
+
+
 def test_fast_scan_mode_stays_within_two_ulp_of_bwd(api):
     """the hardware-exp/log scans are a measurement aid, not a parity-grade mode: bwd within 2 ulp
     of the CPU path, and a posterior may leave the 1e-3 bar (only a loose bound is asserted)"""
