@@ -201,7 +201,7 @@ def main():
                          "main result (0 = skip)")
     ap.add_argument("--no-five-columns", action="store_true",
                     help="skip the side measurement on the same scores with five columns per state (C = 5 * 4^state_len)")
-    ap.add_argument("--overlap-steps", type=int, default=5,
+    ap.add_argument("--overlap-steps", type=int, default=15,
                     help="calls per gpubuf of the two-batches-in-flight side measurement (0 = skip)")
     ap.add_argument("--copy-mib", type=int, default=1024,
                     help="size of the device copy whose GB/s is reported beside the 8 TB/s peak (0 = skip)")
