@@ -2,11 +2,13 @@
  * Host side of the MI355X decoder: the public openfish entry points and the
  * stage-level C-ABI, in C, above the kernel launchers of kernels.h.
  *
- * One decode is   scans + posterior (one kernel) -> beam search -> sequence   on one stream, or,
- * for very large batches and on request,   bwd scan -> { beam search || fwd+posterior scan } ->
- * sequence   on two (the beam search needs only scores and bwd, the posterior only feeds the
- * quality stage, reference src/beam_search.c:193,450).  Errors follow the reference convention (reference
- * src/hip_utils.h:11-28, src/error.h:44-72): message on stderr, then exit.
+ * One decode is   bwd scan -> { beam search || fwd+posterior scan } -> sequence   on two streams
+ * (the beam search needs only scores and bwd, the posterior only feeds the quality stage, reference
+ * src/beam_search.c:193,450) while the beam search leaves the machine idle, and   scans + posterior
+ * (one kernel) -> { beam search || per-state sums of posteriors } -> sequence   for larger batches and
+ * 1024 states; every call chooses unless the gpubuf says which (split_by_default).  The sequence stage
+ * writes bases and qualities into pinned host memory itself.  Errors follow the reference convention
+ * (reference src/hip_utils.h:11-28, src/error.h:44-72): message on stderr, then exit.
  */
 #include <errno.h>
 #include <float.h>
